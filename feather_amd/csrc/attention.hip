@@ -1,0 +1,320 @@
+// Non-causal flash-attention forward on FP8-packed Q/K/V (prefill).
+//
+// Work split.  One workgroup (4 waves) owns a tile of 64*QB queries of one
+// head; each wave owns 16*QB of them for the whole key loop.  Keys/values are
+// streamed in tiles of BN keys: the PACKED tile is fetched from global memory
+// into registers one tile ahead (so HBM/L2 latency overlaps the MFMA work of
+// the current tile), decoded to fp16 on its way into LDS, and read from LDS as
+// MFMA operands by all four waves.
+//
+// Matrix cores.  Everything is computed transposed so that one lane keeps one
+// query for the whole kernel:
+//     S^T[key, q] = K[key, :] . Q[q, :]     v_mfma_f32_16x16x32_f16, A = K tile
+//     O^T[dd, q] += V^T[dd, key] P^T[key, q]  same instruction, A = V^T tile
+// In the 16x16 accumulator layout lane l holds column l % 16 (the query) and
+// rows 4 * (l / 16) + {0..3}; the B operand of the next MFMA wants, for the
+// same column, 8 consecutive k-slots per lane.  The two layouts are matched by
+// permuting the key order in which V^T is written to LDS, so the softmax
+// output feeds the second MFMA straight from registers: no shuffle, no LDS
+// round trip for P.  Row maxima need one exchange across the 4 lanes that
+// share a query (two ds_swizzle/bpermute steps); row sums stay per lane until
+// the epilogue.
+//
+// Numerics follow the reference kernel (feather/routines/attention.py:24-108):
+// fp16 x fp16 products accumulated in fp32, scores scaled in fp32, online
+// softmax in fp32 (computed as 2^x with log2(e) folded into the scale), P
+// rounded to fp16 before P.V, fp32 output.
+#include "common.h"
+
+namespace feather {
+
+constexpr int kAttnThreads = 256;
+
+__device__ __forceinline__ float4_t mfma16(half8_t a, half8_t b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// 8 codes (two packed words) -> 8 fp16
+template <int MODE>
+__device__ __forceinline__ half8_t dec8(uint32_t w0, uint32_t w1) {
+    u32x4 r;
+    uint32_t a, b;
+    dec_word<MODE>(w0, a, b);
+    r.x = a; r.y = b;
+    dec_word<MODE>(w1, a, b);
+    r.z = a; r.w = b;
+    return __builtin_bit_cast(half8_t, r);
+}
+
+__device__ __forceinline__ float xor_lane(float x, int mask) {
+    return __shfl_xor(x, mask, kWave);
+}
+
+template <int D, int MODE, int QB, int BN>
+__global__ __launch_bounds__(kAttnThreads) void flash_attn_kernel(
+    const uint32_t *__restrict__ q, const uint32_t *__restrict__ k, const uint32_t *__restrict__ v,
+    float *__restrict__ out, int L, int n_heads, int kv_group, int tiles_per_head, float scale_log2e,
+    int keys_scored, int mask_tail) {
+    constexpr int DW = D / 4;              // packed words per row
+    constexpr int KS = D + 8;              // fp16 per K row in LDS (16 B pad against bank conflicts)
+    constexpr int VS = BN + 8;             // fp16 per V^T row in LDS
+    constexpr int QT = 64 * QB;            // queries per workgroup
+    constexpr int NU = BN * D / 16 / kAttnThreads;  // 16-code units per thread per tile
+    static_assert(NU >= 1, "tile too small for 256 threads");
+    constexpr int KB16 = BN / 16, KB32 = BN / 32, DB = D / 16, STEPS = D / 32;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    _Float16 *k_lds = reinterpret_cast<_Float16 *>(smem);
+    _Float16 *vt_lds = k_lds + BN * KS;
+
+    // XCD-aware block mapping: consecutive workgroup ids go round-robin over the 8
+    // XCDs (each with its own L2); remap so that an XCD works through a contiguous
+    // range of (head, tile) pairs and the K/V of a head stay in one L2.
+    int bid = blockIdx.x;
+    const int total = gridDim.x;
+    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
+    const int head = bid / tiles_per_head;
+    const int tile = bid % tiles_per_head;
+    const int kv_head = head / kv_group;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 15, kb = lane >> 4;
+    const int q0 = tile * QT + wave * (16 * QB);
+
+    const uint32_t *qh = q + (int64_t)head * L * DW;
+    const uint32_t *kh = k + (int64_t)kv_head * L * DW;
+    const uint32_t *vh = v + (int64_t)kv_head * L * DW;
+
+    // ---- Q fragments (B operand of S^T), resident in registers
+    half8_t qf[QB][STEPS];
+#pragma unroll
+    for (int b = 0; b < QB; b++) {
+        int row = q0 + 16 * b + j;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            u32x2 w = u32x2{0, 0};
+            if (row < L) w = *reinterpret_cast<const u32x2 *>(qh + (int64_t)row * DW + 8 * s + 2 * kb);
+            qf[b][s] = dec8<MODE>(w.x, w.y);
+        }
+    }
+
+    float4_t o[QB][DB];
+    float m_run[QB], l_run[QB];
+#pragma unroll
+    for (int b = 0; b < QB; b++) {
+        m_run[b] = -INFINITY;
+        l_run[b] = 0.f;
+#pragma unroll
+        for (int d = 0; d < DB; d++) o[b][d] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // ---- register staging of the next packed K / V tile
+    u32x4 kreg[NU];
+    uint32_t vreg[NU][4];
+    auto prefetch = [&](int key0) {
+#pragma unroll
+        for (int i = 0; i < NU; i++) {
+            int u = tid + kAttnThreads * i;
+            int key = key0 + u / (D / 16), c16 = u % (D / 16);
+            kreg[i] = u32x4{0, 0, 0, 0};
+            if (key < L) kreg[i] = *reinterpret_cast<const u32x4 *>(kh + (int64_t)key * DW + 4 * c16);
+            int ddw = u % DW, kg = u / DW;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                int vkey = key0 + 4 * kg + r;
+                vreg[i][r] = vkey < L ? vh[(int64_t)vkey * DW + ddw] : 0u;
+            }
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < NU; i++) {
+            int u = tid + kAttnThreads * i;
+            // K: 16 codes of one key -> 16 fp16, row-major [key][d]
+            int key = u / (D / 16), c16 = u % (D / 16);
+            half8_t lo = dec8<MODE>(kreg[i].x, kreg[i].y), hi = dec8<MODE>(kreg[i].z, kreg[i].w);
+            half8_t *kd = reinterpret_cast<half8_t *>(k_lds + key * KS + 16 * c16);
+            kd[0] = lo;
+            kd[1] = hi;
+            // V: 4 keys x 4 dims -> V^T[dd][pos], key order permuted inside each
+            // group of 32 so that slot (kb, 4a + r) holds key 16a + 4kb + r
+            int ddw = u % DW, kg = u / DW;
+            int ko = 4 * kg, o32 = ko & 31;
+            int pos = (ko & ~31) + ((o32 & 15) >> 2) * 8 + (o32 >> 4) * 4;
+            uint32_t lo2[4], hi2[4];
+            if constexpr (MODE == FEATHER_E5M2) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    // halfs (key r, key r+1) of dim 4*ddw + c: byte c of each word, placed as the high byte
+                    uint32_t sel = 0x000c000cu | ((uint32_t)c << 8) | ((uint32_t)(4 + c) << 24);
+                    lo2[c] = perm(vreg[i][1], vreg[i][0], sel);
+                    hi2[c] = perm(vreg[i][3], vreg[i][2], sel);
+                }
+            } else {
+                uint32_t p01[4], p23[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) dec_word<MODE>(vreg[i][r], p01[r], p23[r]);
+                lo2[0] = perm(p01[1], p01[0], 0x05040100u); hi2[0] = perm(p01[3], p01[2], 0x05040100u);
+                lo2[1] = perm(p01[1], p01[0], 0x07060302u); hi2[1] = perm(p01[3], p01[2], 0x07060302u);
+                lo2[2] = perm(p23[1], p23[0], 0x05040100u); hi2[2] = perm(p23[3], p23[2], 0x05040100u);
+                lo2[3] = perm(p23[1], p23[0], 0x07060302u); hi2[3] = perm(p23[3], p23[2], 0x07060302u);
+            }
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                *reinterpret_cast<u32x2 *>(vt_lds + (4 * ddw + c) * VS + pos) = u32x2{lo2[c], hi2[c]};
+        }
+    };
+
+    prefetch(0);
+    for (int key0 = 0; key0 < keys_scored; key0 += BN) {
+        __syncthreads();  // every wave is done reading the previous tile
+        stage();
+        __syncthreads();
+        if (key0 + BN < keys_scored) prefetch(key0 + BN);
+
+        // ---- S^T = K Q^T for this wave's queries
+        float4_t s[QB][KB16];
+#pragma unroll
+        for (int c = 0; c < KB16; c++) {
+#pragma unroll
+            for (int b = 0; b < QB; b++) s[b][c] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int st = 0; st < STEPS; st++) {
+                half8_t kf = *reinterpret_cast<const half8_t *>(k_lds + (16 * c + j) * KS + 32 * st + 8 * kb);
+#pragma unroll
+                for (int b = 0; b < QB; b++) s[b][c] = mfma16(kf, qf[b][st], s[b][c]);
+            }
+        }
+
+        // ---- online softmax, one query per lane column
+        half8_t pf[QB][KB32];
+#pragma unroll
+        for (int b = 0; b < QB; b++) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int c = 0; c < KB16; c++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float x = s[b][c][r] * scale_log2e;
+                    if (mask_tail && key0 + 16 * c + 4 * kb + r >= L) x = -INFINITY;
+                    s[b][c][r] = x;
+                    mx = fmaxf(mx, x);
+                }
+            mx = fmaxf(mx, xor_lane(mx, 16));
+            mx = fmaxf(mx, xor_lane(mx, 32));
+            float m_new = fmaxf(m_run[b], mx);
+            float alpha = __builtin_amdgcn_exp2f(m_run[b] - m_new);
+            m_run[b] = m_new;
+            float rs = 0.f;
+#pragma unroll
+            for (int t = 0; t < KB32; t++) {
+                half8_t p8;
+#pragma unroll
+                for (int a = 0; a < 2; a++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float e = __builtin_amdgcn_exp2f(s[b][2 * t + a][r] - m_new);
+                        rs += e;
+                        p8[4 * a + r] = (_Float16)e;  // round to nearest even, as P.to(fp16)
+                    }
+                pf[b][t] = p8;
+            }
+            l_run[b] = l_run[b] * alpha + rs;
+#pragma unroll
+            for (int d = 0; d < DB; d++) o[b][d] *= alpha;
+        }
+
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int t = 0; t < KB32; t++)
+#pragma unroll
+            for (int d = 0; d < DB; d++) {
+                half8_t vf = *reinterpret_cast<const half8_t *>(vt_lds + (16 * d + j) * VS + 32 * t + 8 * kb);
+#pragma unroll
+                for (int b = 0; b < QB; b++) o[b][d] = mfma16(vf, pf[b][t], o[b][d]);
+            }
+    }
+
+    // ---- epilogue: finish the row sums, normalise, store [q][dd]
+    float *oh = out + (int64_t)head * L * D;
+#pragma unroll
+    for (int b = 0; b < QB; b++) {
+        float l = l_run[b];
+        l += xor_lane(l, 16);
+        l += xor_lane(l, 32);
+        int row = q0 + 16 * b + j;
+        if (row < L) {
+#pragma unroll
+            for (int d = 0; d < DB; d++) {
+                float4_t r = o[b][d] / l;
+                *reinterpret_cast<float4_t *>(oh + (int64_t)row * D + 16 * d + 4 * kb) = r;
+            }
+        }
+    }
+}
+
+template <int D, int MODE, int QB, int BN>
+static int launch_attn(const void *q, const void *k, const void *v, void *out, int64_t n_heads, int64_t L,
+                       int64_t kv_group, float scale, int tail, hipStream_t s) {
+    constexpr int QT = 64 * QB;
+    constexpr size_t lds = (size_t)(BN * (D + 8) + D * (BN + 8)) * 2;
+    int tiles = (int)((L + QT - 1) / QT);
+    int64_t blocks = tiles * n_heads;
+    FEATHER_CHECK(blocks < (1ll << 31), FEATHER_ESHAPE, "feather_flash_attn_fp8: grid too large");
+    // the reference scores whole 64-key tiles (zero rows past L); otherwise only tiles of BN up to L
+    int64_t keys_scored = tail == FEATHER_TAIL_REFERENCE ? (L + 63) / 64 * 64 : (L + BN - 1) / BN * BN;
+    auto kern = flash_attn_kernel<D, MODE, QB, BN>;
+    if (lds > 64 * 1024) {
+        static bool attr_set = false;  // per instantiation
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            FEATHER_CHECK(e == hipSuccess, FEATHER_ELAUNCH, "feather_flash_attn_fp8: cannot raise LDS limit: %s",
+                          hipGetErrorString(e));
+            attr_set = true;
+        }
+    }
+    const float log2e = 1.4426950408889634f;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kAttnThreads), lds, s, (const uint32_t *)q,
+                       (const uint32_t *)k, (const uint32_t *)v, (float *)out, (int)L, (int)n_heads, (int)kv_group,
+                       tiles, scale * log2e, (int)keys_scored, tail == FEATHER_TAIL_MASK ? 1 : 0);
+    return check_launch("feather_flash_attn_fp8");
+}
+
+template <int MODE>
+static int dispatch_attn(const void *q, const void *k, const void *v, void *out, int64_t n_heads, int64_t L, int64_t d,
+                         int64_t kv_group, float scale, int tail, hipStream_t s) {
+    switch (d) {
+        case 64: return launch_attn<64, MODE, 2, 64>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+        case 128: return launch_attn<128, MODE, 2, 64>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+        case 256: return launch_attn<256, MODE, 1, 32>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+        case 512: return launch_attn<512, MODE, 1, 32>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+    }
+    set_error("feather_flash_attn_fp8: head dim %lld not supported (64, 128, 256, 512)", (long long)d);
+    return FEATHER_ESHAPE;
+}
+
+}  // namespace feather
+
+using namespace feather;
+
+extern "C" int feather_flash_attn_fp8(const void *q, const void *k, const void *v, void *out_f32, int64_t n_heads,
+                                      int64_t L, int64_t d, int64_t kv_group, int mode, float scale, int tail,
+                                      void *stream) {
+    FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE,
+                  "feather_flash_attn_fp8: mode %d not supported", mode);
+    FEATHER_CHECK(tail == FEATHER_TAIL_MASK || tail == FEATHER_TAIL_REFERENCE, FEATHER_EINVAL,
+                  "feather_flash_attn_fp8: bad tail flag %d", tail);
+    FEATHER_CHECK(n_heads >= 0 && L >= 0 && d > 0, FEATHER_EINVAL, "feather_flash_attn_fp8: negative shape");
+    FEATHER_CHECK(kv_group >= 1 && n_heads % kv_group == 0, FEATHER_ESHAPE,
+                  "feather_flash_attn_fp8: n_heads=%lld is not a multiple of kv_group=%lld", (long long)n_heads,
+                  (long long)kv_group);
+    FEATHER_CHECK(L < (1ll << 30), FEATHER_ESHAPE, "feather_flash_attn_fp8: sequence too long");
+    if (n_heads == 0 || L == 0) return FEATHER_OK;
+    FEATHER_CHECK(q && k && v && out_f32, FEATHER_EINVAL, "feather_flash_attn_fp8: null pointer");
+    FEATHER_CHECK(aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out_f32, 16), FEATHER_EINVAL,
+                  "feather_flash_attn_fp8: pointers must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    if (mode == FEATHER_E5M2) return dispatch_attn<FEATHER_E5M2>(q, k, v, out_f32, n_heads, L, d, kv_group, scale, tail, s);
+    return dispatch_attn<FEATHER_E4M3>(q, k, v, out_f32, n_heads, L, d, kv_group, scale, tail, s);
+}

@@ -1,0 +1,142 @@
+// Shared device/host helpers for the gfx950 kernels: FP8 decode in registers,
+// wave64 reductions, error reporting.  Wave size is 64 everywhere.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/feather_hip.h"
+
+namespace feather {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------- host side
+
+void set_error(const char *fmt, ...);
+
+#define FEATHER_CHECK(cond, code, ...)      \
+    do {                                    \
+        if (!(cond)) {                      \
+            feather::set_error(__VA_ARGS__); \
+            return (code);                  \
+        }                                   \
+    } while (0)
+
+inline int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+        return FEATHER_ELAUNCH;
+    }
+    return FEATHER_OK;
+}
+
+inline bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// ---------------------------------------------------------------- bit casts
+
+__device__ __forceinline__ half2_t as_half2(uint32_t x) { return __builtin_bit_cast(half2_t, x); }
+__device__ __forceinline__ uint32_t as_u32(half2_t x) { return __builtin_bit_cast(uint32_t, x); }
+__device__ __forceinline__ float as_float(uint32_t x) { return __builtin_bit_cast(float, x); }
+__device__ __forceinline__ uint32_t as_u32(float x) { return __builtin_bit_cast(uint32_t, x); }
+
+// v_perm_b32: result byte i = byte sel[i] of the 8-byte value {hi, lo}
+// (0..3 = lo bytes, 4..7 = hi bytes, 0x0c = constant 0x00).
+__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) {
+    return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+// Streaming (non-temporal) 128-bit accesses: data touched once should not
+// displace the re-used vector / K/V tiles from L2.
+__device__ __forceinline__ u32x4 load_nt128(const void *p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+}
+__device__ __forceinline__ void store_nt128(void *p, u32x4 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
+}
+__device__ __forceinline__ void store_nt64(void *p, u32x2 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x2 *>(p));
+}
+
+// ---------------------------------------------------------------- FP8 -> fp16 pairs
+
+// E5M2 code c is the fp16 with bits c << 8 (reference gemv.py:31-58): decoding a
+// word is byte placement.  p01 = (c0, c1), p23 = (c2, c3) as packed fp16.
+__device__ __forceinline__ void dec_e5m2_word(uint32_t w, uint32_t &p01, uint32_t &p23) {
+    p01 = perm(w, w, 0x010c000cu);
+    p23 = perm(w, w, 0x030c020cu);
+}
+
+// E4M3 code -> fp16 bits sign | (e ? e + 8 : 0) << 10 | m << 7 (reference
+// gemv.py:83-88), four codes at a time with byte-parallel integer arithmetic:
+//   high byte  H = sign | ((c >> 1) & 0x3F) + (e > 0 ? 0x20 : 0)
+//   low byte   L = (c & 1) << 7
+// (e > 0) is bit 7 of (c & 0x78) + 0x7F; no byte ever carries into the next.
+__device__ __forceinline__ void dec_e4m3_word(uint32_t w, uint32_t &p01, uint32_t &p23) {
+    uint32_t nz = (w & 0x78787878u) + 0x7F7F7F7Fu;
+    uint32_t bias = (nz >> 2) & 0x20202020u;
+    uint32_t mag = ((w >> 1) & 0x3F3F3F3Fu) + bias;
+    uint32_t hi = (w & 0x80808080u) | mag;
+    uint32_t lo = (w << 7) & 0x80808080u;
+    p01 = perm(hi, lo, 0x05010400u);
+    p23 = perm(hi, lo, 0x07030602u);
+}
+
+template <int MODE>
+__device__ __forceinline__ void dec_word(uint32_t w, uint32_t &p01, uint32_t &p23) {
+    if constexpr (MODE == FEATHER_E5M2) dec_e5m2_word(w, p01, p23);
+    else dec_e4m3_word(w, p01, p23);
+}
+
+// E4M3fn code -> fp16 bits with the exact (OCP) value; used by the unpack
+// kernel for the CPU-API semantics (reference fp8.py:381-391).
+__device__ __forceinline__ uint32_t dec_e4m3_ieee_bits(uint32_t c) {
+    uint32_t sign = (c & 0x80u) << 8;
+    uint32_t e = (c >> 3) & 0xFu, m = c & 7u;
+    if ((c & 0x7Fu) == 0x7Fu) return sign | 0x7E00u;
+    if (e) return sign | ((e + 8u) << 10) | (m << 7);
+    if (!m) return sign;
+    uint32_t lead = m >= 4 ? 2u : (m >= 2 ? 1u : 0u);
+    return sign | ((6u + lead) << 10) | ((m << (10u - lead)) & 0x3FFu);
+}
+
+// acc += a.x * b.x + a.y * b.y with fp32 accumulation (v_dot2_f32_f16); the
+// fp16 x fp16 products are exact in fp32.
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2(as_half2(a), as_half2(b), acc, false);
+}
+
+// ---------------------------------------------------------------- wave64 reductions
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+    return as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)as_u32(x), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the 64 lanes of a wave; every lane of row 0 (lanes 0..15) gets the
+// total.  quad_perm / row_half_mirror / row_mirror fold each 16-lane row, then
+// the four row sums are read with v_readlane.
+__device__ __forceinline__ float wave_sum(float x) {
+    x += dpp_mov<0xB1>(x);   // quad_perm [1,0,3,2]
+    x += dpp_mov<0x4E>(x);   // quad_perm [2,3,0,1]
+    x += dpp_mov<0x141>(x);  // row_half_mirror
+    x += dpp_mov<0x140>(x);  // row_mirror
+    float r0 = as_float((uint32_t)__builtin_amdgcn_readlane((int)as_u32(x), 0));
+    float r1 = as_float((uint32_t)__builtin_amdgcn_readlane((int)as_u32(x), 16));
+    float r2 = as_float((uint32_t)__builtin_amdgcn_readlane((int)as_u32(x), 32));
+    float r3 = as_float((uint32_t)__builtin_amdgcn_readlane((int)as_u32(x), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }
+
+}  // namespace feather

@@ -1,0 +1,205 @@
+// Packed-FP8 GEMV: out[r] = sum_k dec(m[r,k]) * dec(v[k]), fp32 accumulate.
+//
+// The kernel is a pure HBM stream of the matrix (1 byte per element); the
+// vector (K bytes) is decoded ONCE per workgroup into LDS as fp16 and re-used
+// by every row the workgroup owns.
+//
+//   * one wave owns RPW rows at a time; a lane reads 16 consecutive codes
+//     (one 128-bit non-temporal load) per row per step, so a wave-load covers
+//     1 KiB of contiguous row bytes; U steps are issued back to back to keep
+//     RPW * U loads in flight per lane;
+//   * decode is register-only: E5M2 is byte placement (v_perm_b32), E4M3 is
+//     byte-parallel integer arithmetic on four codes at a time;
+//   * multiply-accumulate is v_dot2_f32_f16 (two exact fp16 x fp16 products
+//     added into an fp32 accumulator);
+//   * the RPW row sums are folded across the wave with DPP.
+//
+// A workgroup takes a contiguous range of rows so the vector decode is
+// amortised; ranges are sized so that the grid is a few workgroups per CU.
+#include "common.h"
+
+namespace feather {
+
+constexpr int kGemvThreads = 256;
+constexpr int kGemvWaves = kGemvThreads / kWave;
+constexpr int kMaxChunk = 32768;  // codes of the vector held in LDS at once (64 KiB as fp16)
+
+// Decode `n_words` packed words of the vector into LDS as fp16 (natural
+// order) and zero the padding up to `lds_halfs`.
+template <int MODE>
+__device__ __forceinline__ void stage_vector(const uint32_t *__restrict__ v, uint32_t *lds32, int n_words,
+                                             int lds_words) {
+    for (int i = threadIdx.x; i < lds_words; i += kGemvThreads) {
+        uint32_t p01 = 0, p23 = 0;
+        if (i < n_words) dec_word<MODE>(v[i], p01, p23);
+        reinterpret_cast<u32x2 *>(lds32)[i] = u32x2{p01, p23};
+    }
+}
+
+// 16 codes (one uint4) of a row against the matching 16 fp16 of the vector.
+template <int MODE>
+__device__ __forceinline__ float mac16(const u32x4 &a, const u32x4 &x0, const u32x4 &x1, float acc) {
+    uint32_t p, q;
+    dec_word<MODE>(a.x, p, q);
+    acc = dot2(p, x0.x, acc);
+    acc = dot2(q, x0.y, acc);
+    dec_word<MODE>(a.y, p, q);
+    acc = dot2(p, x0.z, acc);
+    acc = dot2(q, x0.w, acc);
+    dec_word<MODE>(a.z, p, q);
+    acc = dot2(p, x1.x, acc);
+    acc = dot2(q, x1.y, acc);
+    dec_word<MODE>(a.w, p, q);
+    acc = dot2(p, x1.z, acc);
+    acc = dot2(q, x1.w, acc);
+    return acc;
+}
+
+// Fast path: rows are 16-byte aligned (K % 16 == 0, base aligned).
+//   m        matrix, row stride K bytes
+//   v        vector words for columns [k0, k0 + kc)
+//   k0, kc   column chunk handled by this launch (kc <= kMaxChunk, kc % 16 == 0)
+//   accumulate  add to out instead of overwriting (later chunks)
+template <int MODE, int RPW, int U>
+__global__ __launch_bounds__(kGemvThreads) void gemv_fp8_kernel(const uint8_t *__restrict__ m,
+                                                               const uint32_t *__restrict__ v,
+                                                               float *__restrict__ out, int M, int64_t K, int k0,
+                                                               int kc, int rows_per_wg, int accumulate) {
+    extern __shared__ uint32_t lds32[];  // fp16 vector chunk, padded to a multiple of 1024 * U halfs
+    constexpr int kStep = kWave * 16;    // codes per wave-load
+    const int kc_pad = (kc + kStep * U - 1) / (kStep * U) * (kStep * U);
+    stage_vector<MODE>(v, lds32, kc / 4, kc_pad / 4);
+    __syncthreads();
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x / kWave;
+    const int row_begin = blockIdx.x * rows_per_wg;
+    const int row_end = min(row_begin + rows_per_wg, M);
+    const u32x4 *lds128 = reinterpret_cast<const u32x4 *>(lds32);
+
+    for (int r0 = row_begin + wave * RPW; r0 < row_end; r0 += kGemvWaves * RPW) {
+        float acc[RPW];
+        const uint8_t *rowp[RPW];
+#pragma unroll
+        for (int r = 0; r < RPW; r++) {
+            acc[r] = 0.f;
+            int row = min(r0 + r, M - 1);  // clamp: surplus rows re-read the last row, result dropped
+            rowp[r] = m + (int64_t)row * K + k0 + lane * 16;
+        }
+        for (int c = 0; c < kc; c += kStep * U) {
+            u32x4 a[RPW][U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                int col = c + u * kStep + lane * 16;
+                bool ok = col < kc;
+#pragma unroll
+                for (int r = 0; r < RPW; r++) {
+                    a[r][u] = u32x4{0, 0, 0, 0};
+                    if (ok) a[r][u] = load_nt128(rowp[r] + c + u * kStep);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                int col = c + u * kStep + lane * 16;   // < kc_pad: LDS is padded with zeros
+                u32x4 x0 = lds128[col / 8];
+                u32x4 x1 = lds128[col / 8 + 1];
+#pragma unroll
+                for (int r = 0; r < RPW; r++) acc[r] = mac16<MODE>(a[r][u], x0, x1, acc[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; r++) {
+            float s = wave_sum(acc[r]);
+            if (lane == 0 && r0 + r < row_end) {
+                if (accumulate) s += out[r0 + r];
+                out[r0 + r] = s;
+            }
+        }
+    }
+}
+
+// Generic path: any K % 4 == 0 and 4-byte aligned rows; one word per lane per
+// step.  Used for shapes whose rows are not 16-byte aligned.
+template <int MODE>
+__global__ __launch_bounds__(kGemvThreads) void gemv_fp8_generic_kernel(const uint32_t *__restrict__ m,
+                                                                       const uint32_t *__restrict__ v,
+                                                                       float *__restrict__ out, int M, int64_t n_col) {
+    const int lane = lane_id();
+    const int wave = threadIdx.x / kWave;
+    for (int row = blockIdx.x * kGemvWaves + wave; row < M; row += gridDim.x * kGemvWaves) {
+        const uint32_t *rp = m + (int64_t)row * n_col;
+        float acc = 0.f;
+        for (int64_t j = lane; j < n_col; j += kWave) {
+            uint32_t p, q, x, y;
+            dec_word<MODE>(rp[j], p, q);
+            dec_word<MODE>(v[j], x, y);
+            acc = dot2(p, x, acc);
+            acc = dot2(q, y, acc);
+        }
+        float s = wave_sum(acc);
+        if (lane == 0) out[row] = s;
+    }
+}
+
+__global__ void fill_zero_kernel(float *p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.f;
+}
+
+template <int MODE>
+static int launch_gemv(const void *m, const void *v, float *out, int64_t M, int64_t K, hipStream_t s) {
+    if (K % 16 != 0 || !aligned(m, 16)) {
+        int64_t blocks = (M + kGemvWaves - 1) / kGemvWaves;
+        if (blocks > 256 * 8) blocks = 256 * 8;
+        hipLaunchKernelGGL((gemv_fp8_generic_kernel<MODE>), dim3((unsigned)blocks), dim3(kGemvThreads), 0, s,
+                           (const uint32_t *)m, (const uint32_t *)v, out, (int)M, K / 4);
+        return check_launch("feather_gemv_fp8");
+    }
+    constexpr int RPW = 2, U = 4;
+    constexpr int kStep = kWave * 16;
+    // rows per workgroup: aim at ~4 workgroups per CU (256 CUs) so the vector
+    // decode (K bytes from L2 per workgroup) stays a few percent of the matrix
+    // bytes the workgroup streams, in multiples of the 8 rows one pass covers.
+    int64_t rows_per_wg = (M + 1023) / 1024;
+    rows_per_wg = (rows_per_wg + kGemvWaves * RPW - 1) / (kGemvWaves * RPW) * (kGemvWaves * RPW);
+    int64_t blocks = (M + rows_per_wg - 1) / rows_per_wg;
+    for (int64_t k0 = 0; k0 < K; k0 += kMaxChunk) {
+        int kc = (int)((K - k0) < kMaxChunk ? (K - k0) : kMaxChunk);
+        int kc_pad = (kc + kStep * U - 1) / (kStep * U) * (kStep * U);
+        size_t lds = (size_t)kc_pad * 2;
+        hipLaunchKernelGGL((gemv_fp8_kernel<MODE, RPW, U>), dim3((unsigned)blocks), dim3(kGemvThreads), lds, s,
+                           (const uint8_t *)m, (const uint32_t *)v + k0 / 4, out, (int)M, K, (int)k0, kc,
+                           (int)rows_per_wg, k0 > 0 ? 1 : 0);
+        int rc = check_launch("feather_gemv_fp8");
+        if (rc != FEATHER_OK) return rc;
+    }
+    return FEATHER_OK;
+}
+
+}  // namespace feather
+
+using namespace feather;
+
+extern "C" int feather_gemv_fp8(const void *m, const void *v, void *out_f32, int64_t M, int64_t K, int mode,
+                                void *stream) {
+    FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE, "feather_gemv_fp8: mode %d not supported",
+                  mode);
+    FEATHER_CHECK(M >= 0 && K >= 0, FEATHER_EINVAL, "feather_gemv_fp8: negative shape");
+    FEATHER_CHECK(K % 4 == 0, FEATHER_ESHAPE,
+                  "feather_gemv_fp8: K=%lld is not a multiple of 4 (rows would straddle packed words)", (long long)K);
+    FEATHER_CHECK(M < (1ll << 31) && K < (1ll << 31), FEATHER_ESHAPE, "feather_gemv_fp8: shape too large");
+    if (M == 0) return FEATHER_OK;
+    FEATHER_CHECK(out_f32, FEATHER_EINVAL, "feather_gemv_fp8: null out");
+    FEATHER_CHECK(aligned(out_f32, 4), FEATHER_EINVAL, "feather_gemv_fp8: misaligned out");
+    if (K == 0) {
+        // empty rows sum to zero; a fill kernel (not a memset node) keeps the call graph-capturable
+        int64_t blocks = (M + 255) / 256;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0,
+                           (hipStream_t)stream, (float *)out_f32, M);
+        return check_launch("feather_gemv_fp8");
+    }
+    FEATHER_CHECK(m && v, FEATHER_EINVAL, "feather_gemv_fp8: null pointer");
+    FEATHER_CHECK(aligned(m, 4) && aligned(v, 4), FEATHER_EINVAL, "feather_gemv_fp8: misaligned pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (mode == FEATHER_E5M2) return launch_gemv<FEATHER_E5M2>(m, v, (float *)out_f32, M, K, s);
+    return launch_gemv<FEATHER_E4M3>(m, v, (float *)out_f32, M, K, s);
+}

@@ -1,0 +1,292 @@
+// Pack / unpack kernels: fp16 -> four FP8 codes per 32-bit word and back, and
+// the two-fp16-per-word container.  All are pure streaming kernels bound by HBM
+// bandwidth (pack: 2 B in + 1 B out per element; unpack to fp32: 1 B in + 4 B
+// out), so the work is laid out for full-width coalesced accesses: one lane
+// converts 16 consecutive elements from two 128-bit loads into one 128-bit
+// store.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.h"
+
+namespace feather {
+
+// ---------------------------------------------------------------- error state
+
+static thread_local char g_err[256] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+// ---------------------------------------------------------------- encoders
+
+// fp16 bits -> E5M2, round to nearest even: E5M2 is the high byte of fp16, so
+// rounding is an integer add on the bit pattern (a carry bumps the exponent,
+// values >= 61440 reach 0x7C = inf).  NaN -> 0x7F | sign.
+__device__ __forceinline__ uint32_t enc_e5m2(uint32_t h) {
+    uint32_t a = h & 0x7FFFu;
+    uint32_t sign = (h >> 8) & 0x80u;
+    uint32_t r = (a + 0x7Fu + ((a >> 8) & 1u)) >> 8;
+    return sign | (a > 0x7C00u ? 0x7Fu : r);
+}
+
+// fp16 bits -> E4M3fn (bias 7, subnormal unit 2^-9, max 448, 0x7F = NaN), RNE.
+// Anything that rounds above 448 (|x| > 464), inf and NaN give 0x7F.
+__device__ __forceinline__ uint32_t enc_e4m3(uint32_t h) {
+    uint32_t a = h & 0x7FFFu;
+    uint32_t sign = (h >> 8) & 0x80u;
+    uint32_t exp = a >> 10;
+    uint32_t code;
+    if (exp >= 9u) {                                  // |x| >= 2^-6: normal in E4M3
+        uint32_t t = a - (8u << 10);                  // rebias 15 -> 7
+        t += 0x3Fu + ((t >> 7) & 1u);                 // RNE on the 7 dropped bits
+        code = min(t >> 7, 0x7Fu);
+    } else {                                          // subnormal target: units of 2^-9
+        uint32_t full = (a & 0x3FFu) | 0x400u;
+        uint32_t sh = 16u - max(exp, 1u);             // 8..15
+        uint32_t q = full >> sh;
+        uint32_t rem = full & ((1u << sh) - 1u);
+        uint32_t half = 1u << (sh - 1u);
+        q += (rem > half || (rem == half && (q & 1u))) ? 1u : 0u;
+        code = exp == 0u ? 0u : q;                    // fp16 subnormals are < 2^-10 -> 0
+    }
+    return sign | code;
+}
+
+template <int MODE, int ROUND>
+__device__ __forceinline__ uint32_t enc(uint32_t h) {
+    if constexpr (ROUND == FEATHER_ROUND_TRUNC) return (h >> 8) & 0xFFu;
+    else if constexpr (MODE == FEATHER_E5M2) return enc_e5m2(h);
+    else return enc_e4m3(h);
+}
+
+// two fp16 (one 32-bit register) -> two codes in bits [0,16)
+template <int MODE, int ROUND>
+__device__ __forceinline__ uint32_t enc_pair(uint32_t hh) {
+    return enc<MODE, ROUND>(hh & 0xFFFFu) | (enc<MODE, ROUND>(hh >> 16) << 8);
+}
+
+// ---------------------------------------------------------------- pack fp8
+
+// Vector body: thread t converts elements [16t, 16t+16) (n16 such groups).
+// Scalar tail: the remaining n - 16*n16 elements, one word per thread with
+// zero padding, handled by the first threads of the grid.
+template <int MODE, int ROUND, bool ALIGNED>
+__global__ __launch_bounds__(256) void pack_fp8_kernel(const uint16_t *__restrict__ src, uint32_t *__restrict__ dst,
+                                                      int64_t n, int64_t n16) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t g = t; g < n16; g += stride) {
+        uint32_t in[8];
+        if constexpr (ALIGNED) {
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(src) + 2 * g;
+            u32x4 a = load_nt128(p), b = load_nt128(p + 1);
+            in[0] = a.x; in[1] = a.y; in[2] = a.z; in[3] = a.w;
+            in[4] = b.x; in[5] = b.y; in[6] = b.z; in[7] = b.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                in[i] = (uint32_t)src[16 * g + 2 * i] | ((uint32_t)src[16 * g + 2 * i + 1] << 16);
+        }
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            w[i] = enc_pair<MODE, ROUND>(in[2 * i]) | (enc_pair<MODE, ROUND>(in[2 * i + 1]) << 16);
+        if constexpr (ALIGNED) {
+            store_nt128(reinterpret_cast<u32x4 *>(dst) + g, u32x4{w[0], w[1], w[2], w[3]});
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[4 * g + i] = w[i];
+        }
+    }
+    // tail words
+    int64_t first = 16 * n16;
+    int64_t tail_words = (n - first + 3) / 4;
+    if (t < tail_words) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int64_t idx = first + 4 * t + i;
+            uint32_t h = idx < n ? src[idx] : 0u;
+            w |= enc<MODE, ROUND>(h) << (8 * i);
+        }
+        dst[first / 4 + t] = w;
+    }
+}
+
+template <int MODE, int ROUND>
+static int launch_pack(const void *src, void *dst, int64_t n, hipStream_t s) {
+    int64_t n16 = n / 16;
+    bool al = aligned(src, 16) && aligned(dst, 16);
+    int64_t threads_needed = n16 > 4 ? n16 : 4;
+    int64_t blocks = (threads_needed + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;         // grid-stride beyond 16 workgroups per CU
+    if (blocks < 1) blocks = 1;
+    if (al)
+        hipLaunchKernelGGL((pack_fp8_kernel<MODE, ROUND, true>), dim3((unsigned)blocks), dim3(256), 0, s,
+                           (const uint16_t *)src, (uint32_t *)dst, n, n16);
+    else
+        hipLaunchKernelGGL((pack_fp8_kernel<MODE, ROUND, false>), dim3((unsigned)blocks), dim3(256), 0, s,
+                           (const uint16_t *)src, (uint32_t *)dst, n, n16);
+    return check_launch("feather_pack_fp8");
+}
+
+// ---------------------------------------------------------------- unpack fp8
+
+template <int MODE, int SEM>
+__device__ __forceinline__ void dec_word_sem(uint32_t w, uint32_t &p01, uint32_t &p23) {
+    if constexpr (MODE == FEATHER_E4M3 && SEM == FEATHER_SEM_IEEE) {
+        p01 = dec_e4m3_ieee_bits(w & 0xFFu) | (dec_e4m3_ieee_bits((w >> 8) & 0xFFu) << 16);
+        p23 = dec_e4m3_ieee_bits((w >> 16) & 0xFFu) | (dec_e4m3_ieee_bits(w >> 24) << 16);
+    } else {
+        dec_word<MODE>(w, p01, p23);
+    }
+}
+
+// One word per lane per step: 4-byte loads and 16-byte (fp32) or 8-byte (fp16)
+// stores are both contiguous across the wave.
+template <int MODE, int SEM, int OUT, bool RELU>
+__global__ __launch_bounds__(256) void unpack_fp8_kernel(const uint32_t *__restrict__ src, void *__restrict__ dst,
+                                                        int64_t n_words) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t j = t; j < n_words; j += stride) {
+        uint32_t w = __builtin_nontemporal_load(src + j);
+        uint32_t p01, p23;
+        dec_word_sem<MODE, SEM>(w, p01, p23);
+        half2_t a = as_half2(p01), b = as_half2(p23);
+        if constexpr (RELU) {
+            // max(0, x) as in tl.maximum(0.0, x): a negative or NaN-free compare
+            a.x = a.x > (_Float16)0 ? a.x : (_Float16)0;
+            a.y = a.y > (_Float16)0 ? a.y : (_Float16)0;
+            b.x = b.x > (_Float16)0 ? b.x : (_Float16)0;
+            b.y = b.y > (_Float16)0 ? b.y : (_Float16)0;
+        }
+        if constexpr (OUT == FEATHER_OUT_F32) {
+            store_nt128(reinterpret_cast<u32x4 *>(dst) + j,
+                        u32x4{as_u32((float)a.x), as_u32((float)a.y), as_u32((float)b.x), as_u32((float)b.y)});
+        } else {
+            store_nt64(reinterpret_cast<u32x2 *>(dst) + j, u32x2{as_u32(a), as_u32(b)});
+        }
+    }
+}
+
+template <int MODE, int SEM, int OUT, bool RELU>
+static int launch_unpack(const void *src, void *dst, int64_t n_words, hipStream_t s) {
+    int64_t blocks = (n_words + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL((unpack_fp8_kernel<MODE, SEM, OUT, RELU>), dim3((unsigned)blocks), dim3(256), 0, s,
+                       (const uint32_t *)src, dst, n_words);
+    return check_launch("feather_unpack_fp8");
+}
+
+template <int MODE, int SEM>
+static int dispatch_unpack(const void *src, void *dst, int64_t n_words, int out_dtype, int relu, hipStream_t s) {
+    if (out_dtype == FEATHER_OUT_F32)
+        return relu ? launch_unpack<MODE, SEM, FEATHER_OUT_F32, true>(src, dst, n_words, s)
+                    : launch_unpack<MODE, SEM, FEATHER_OUT_F32, false>(src, dst, n_words, s);
+    return relu ? launch_unpack<MODE, SEM, FEATHER_OUT_F16, true>(src, dst, n_words, s)
+                : launch_unpack<MODE, SEM, FEATHER_OUT_F16, false>(src, dst, n_words, s);
+}
+
+// ---------------------------------------------------------------- fp16 container
+
+// word j = src[2j] | src[2j+1] << 16, odd tail padded with +0.  On a
+// little-endian device this is a copy with a zeroed last half-word.
+__global__ __launch_bounds__(256) void pack_fp16_kernel(const uint16_t *__restrict__ src, uint32_t *__restrict__ dst,
+                                                       int64_t n) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t nw = (n + 1) / 2;
+    for (int64_t j = t; j < nw; j += stride) {
+        uint32_t lo = src[2 * j];
+        uint32_t hi = 2 * j + 1 < n ? src[2 * j + 1] : 0u;
+        dst[j] = lo | (hi << 16);
+    }
+}
+
+__global__ __launch_bounds__(256) void unpack_fp16_kernel(const uint32_t *__restrict__ src, uint16_t *__restrict__ dst,
+                                                         int64_t n_words) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t j = t; j < n_words; j += stride) {
+        uint32_t w = src[j];
+        dst[2 * j] = (uint16_t)(w & 0xFFFFu);
+        dst[2 * j + 1] = (uint16_t)(w >> 16);
+    }
+}
+
+}  // namespace feather
+
+using namespace feather;
+
+extern "C" int feather_version(void) { return 100; }
+
+extern "C" const char *feather_last_error(void) { return g_err; }
+
+extern "C" int feather_pack_fp8(const void *src_f16, void *dst_u32, int64_t n, int mode, int rounding, void *stream) {
+    FEATHER_CHECK(n >= 0, FEATHER_EINVAL, "feather_pack_fp8: negative n");
+    FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE, "feather_pack_fp8: mode %d not supported",
+                  mode);
+    FEATHER_CHECK(rounding == FEATHER_ROUND_RNE || rounding == FEATHER_ROUND_TRUNC, FEATHER_EINVAL,
+                  "feather_pack_fp8: bad rounding %d", rounding);
+    FEATHER_CHECK(!(rounding == FEATHER_ROUND_TRUNC && mode != FEATHER_E5M2), FEATHER_EMODE,
+                  "feather_pack_fp8: truncating pack supports E5M2 only");
+    if (n == 0) return FEATHER_OK;
+    FEATHER_CHECK(src_f16 && dst_u32, FEATHER_EINVAL, "feather_pack_fp8: null pointer");
+    FEATHER_CHECK(aligned(src_f16, 2) && aligned(dst_u32, 4), FEATHER_EINVAL, "feather_pack_fp8: misaligned pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (rounding == FEATHER_ROUND_TRUNC) return launch_pack<FEATHER_E5M2, FEATHER_ROUND_TRUNC>(src_f16, dst_u32, n, s);
+    if (mode == FEATHER_E5M2) return launch_pack<FEATHER_E5M2, FEATHER_ROUND_RNE>(src_f16, dst_u32, n, s);
+    return launch_pack<FEATHER_E4M3, FEATHER_ROUND_RNE>(src_f16, dst_u32, n, s);
+}
+
+extern "C" int feather_unpack_fp8(const void *src_u32, void *dst, int64_t n_words, int mode, int semantics,
+                                  int out_dtype, int relu, void *stream) {
+    FEATHER_CHECK(n_words >= 0, FEATHER_EINVAL, "feather_unpack_fp8: negative n_words");
+    FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE,
+                  "feather_unpack_fp8: mode %d not supported", mode);
+    FEATHER_CHECK(semantics == FEATHER_SEM_KERNEL || semantics == FEATHER_SEM_IEEE, FEATHER_EINVAL,
+                  "feather_unpack_fp8: bad semantics %d", semantics);
+    FEATHER_CHECK(out_dtype == FEATHER_OUT_F32 || out_dtype == FEATHER_OUT_F16, FEATHER_EINVAL,
+                  "feather_unpack_fp8: bad out_dtype %d", out_dtype);
+    if (n_words == 0) return FEATHER_OK;
+    FEATHER_CHECK(src_u32 && dst, FEATHER_EINVAL, "feather_unpack_fp8: null pointer");
+    FEATHER_CHECK(aligned(src_u32, 4) && aligned(dst, out_dtype == FEATHER_OUT_F32 ? 16 : 8), FEATHER_EINVAL,
+                  "feather_unpack_fp8: misaligned pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (mode == FEATHER_E5M2) return dispatch_unpack<FEATHER_E5M2, FEATHER_SEM_KERNEL>(src_u32, dst, n_words, out_dtype, relu, s);
+    if (semantics == FEATHER_SEM_IEEE)
+        return dispatch_unpack<FEATHER_E4M3, FEATHER_SEM_IEEE>(src_u32, dst, n_words, out_dtype, relu, s);
+    return dispatch_unpack<FEATHER_E4M3, FEATHER_SEM_KERNEL>(src_u32, dst, n_words, out_dtype, relu, s);
+}
+
+extern "C" int feather_pack_fp16(const void *src_f16, void *dst_u32, int64_t n, void *stream) {
+    FEATHER_CHECK(n >= 0, FEATHER_EINVAL, "feather_pack_fp16: negative n");
+    if (n == 0) return FEATHER_OK;
+    FEATHER_CHECK(src_f16 && dst_u32, FEATHER_EINVAL, "feather_pack_fp16: null pointer");
+    FEATHER_CHECK(aligned(src_f16, 2) && aligned(dst_u32, 4), FEATHER_EINVAL, "feather_pack_fp16: misaligned pointer");
+    int64_t nw = (n + 1) / 2;
+    int64_t blocks = (nw + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    hipLaunchKernelGGL(pack_fp16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t *)src_f16, (uint32_t *)dst_u32, n);
+    return check_launch("feather_pack_fp16");
+}
+
+extern "C" int feather_unpack_fp16(const void *src_u32, void *dst_f16, int64_t n_words, void *stream) {
+    FEATHER_CHECK(n_words >= 0, FEATHER_EINVAL, "feather_unpack_fp16: negative n_words");
+    if (n_words == 0) return FEATHER_OK;
+    FEATHER_CHECK(src_u32 && dst_f16, FEATHER_EINVAL, "feather_unpack_fp16: null pointer");
+    FEATHER_CHECK(aligned(src_u32, 4) && aligned(dst_f16, 2), FEATHER_EINVAL, "feather_unpack_fp16: misaligned pointer");
+    int64_t blocks = (n_words + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    hipLaunchKernelGGL(unpack_fp16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const uint32_t *)src_u32, (uint16_t *)dst_f16, n_words);
+    return check_launch("feather_unpack_fp16");
+}

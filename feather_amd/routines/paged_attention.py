@@ -1,0 +1,63 @@
+"""Single-query attention over a paged FP8 KV cache (decode step).  The reference
+has no paged attention; numerics follow its flash-attention kernel (decode by
+mode, fp32 scores and softmax, P rounded to fp16, fp32 output) and the kernel is
+``csrc/paged_attention.hip``.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import _native as N
+
+__all__ = ["paged_attention_fp8_acc_fp32_gpu"]
+
+
+def paged_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                                     block_tables: torch.Tensor, context_lens: torch.Tensor, *, mode: str = "E5M2",
+                                     scale: float | None = None, max_context_len: int | None = None) -> torch.Tensor:
+    """
+    q             ``[n_seq, n_q_heads, d/4]`` packed words
+    k_cache       ``[n_blocks, n_kv_heads, block_size, d/4]`` packed words (``v_cache`` alike)
+    block_tables  ``[n_seq, max_blocks]`` int32, physical block of each logical block
+    context_lens  ``[n_seq]`` int32
+    Returns float32 ``[n_seq, n_q_heads, d]``.  Query head ``h`` reads KV head
+    ``h // (n_q_heads // n_kv_heads)``.  ``max_context_len`` (default
+    ``max_blocks * block_size``) bounds the context split count without a
+    device-to-host copy of ``context_lens``."""
+    code = N.mode_code(mode)
+    q, k_cache, v_cache = N.as_words(q, "q"), N.as_words(k_cache, "k_cache"), N.as_words(v_cache, "v_cache")
+    if q.dim() != 3 or k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
+        raise ValueError("expected q [n_seq, n_q_heads, d/4] and k_cache/v_cache [n_blocks, n_kv_heads, block_size, d/4]")
+    n_seq, n_q_heads, dw = q.shape
+    n_blocks, n_kv_heads, block_size, dw2 = k_cache.shape
+    if dw != dw2:
+        raise ValueError(f"head dim mismatch: q has {dw} words per head, cache has {dw2}")
+    d = 4 * dw
+    if d not in (64, 128, 256):
+        raise ValueError(f"head dim {d} not supported: 64, 128 or 256")
+    if n_q_heads % n_kv_heads != 0 or n_q_heads // n_kv_heads > 16:
+        raise ValueError(f"n_q_heads={n_q_heads} must be a multiple of n_kv_heads={n_kv_heads} with ratio <= 16")
+    if block_tables.dtype != torch.int32 or context_lens.dtype != torch.int32:
+        raise ValueError("block_tables and context_lens must be int32")
+    if block_tables.dim() != 2 or block_tables.shape[0] != n_seq or context_lens.shape != (n_seq,):
+        raise ValueError("block_tables must be [n_seq, max_blocks] and context_lens [n_seq]")
+    if not (block_tables.is_cuda and context_lens.is_cuda):
+        raise ValueError("block_tables and context_lens must live on the device")
+    block_tables, context_lens = block_tables.contiguous(), context_lens.contiguous()
+    max_blocks = block_tables.shape[1]
+    max_ctx = max_blocks * block_size if max_context_len is None else int(max_context_len)
+    if max_ctx > max_blocks * block_size or max_ctx < 0:
+        raise ValueError(f"max_context_len={max_ctx} exceeds the block table ({max_blocks} x {block_size})")
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    out = torch.empty((n_seq, n_q_heads, d), dtype=torch.float32, device=q.device)
+    nbytes = int(N.lib().feather_paged_attn_scratch_bytes(n_seq, n_q_heads, d, max_ctx))
+    scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        N.check(N.lib().feather_paged_attn_fp8(N.ptr(q), N.ptr(k_cache), N.ptr(v_cache), N.ptr(block_tables),
+                                               N.ptr(context_lens), N.ptr(out), N.ptr(scratch), n_seq, n_q_heads,
+                                               n_kv_heads, d, block_size, max_blocks, max_ctx, code, float(scale),
+                                               N.stream_ptr(q.device)))
+    return out

@@ -1,0 +1,147 @@
+/*
+ * feather_hip.h -- C ABI of libfeather_hip.so: hand-written gfx950 (MI355X)
+ * kernels for the packed-low-precision routines of SuriyaaMM/feather.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless the name says host.  The library
+ *     never allocates, frees or synchronises; outputs and scratch are caller
+ *     owned.  Kernels are enqueued on `stream` (a hipStream_t passed as void*,
+ *     NULL = the default stream) and the call returns at once.
+ *   - Return value: FEATHER_OK (0) or a negative FEATHER_E* code; a message for
+ *     the last failure on the calling thread is available from
+ *     feather_last_error().
+ *   - Packed layout (reference feather/packers/fp8.py:134, fp16.py:39): element
+ *     4j+i of the flattened source is byte i (bits [8i, 8i+8)) of 32-bit word
+ *     j; two fp16 values per word with the first in the low half.
+ *   - `mode`: FEATHER_E5M2 / FEATHER_E4M3.  Decode inside the compute kernels
+ *     follows the reference kernels: E5M2 code c -> fp16 bits c << 8
+ *     (feather/routines/gemv.py:31-58); E4M3 -> sign | (e ? e + 8 : 0) << 10 |
+ *     m << 7 (feather/routines/gemv.py:83-88).
+ *
+ * Each entry point cites the reference interface it replaces (paths relative
+ * to the reference checkout).
+ */
+#ifndef FEATHER_HIP_H
+#define FEATHER_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FEATHER_OK 0
+#define FEATHER_EINVAL (-1)       /* null / misaligned pointer, negative size, bad flag */
+#define FEATHER_EMODE (-2)        /* unknown mode (reference: NotImplementedError, fp8.py:114) */
+#define FEATHER_ESHAPE (-3)       /* shape the kernels do not support (K % 4, head dim, ...) */
+#define FEATHER_ELAUNCH (-4)      /* hipGetLastError() after a launch */
+
+#define FEATHER_E5M2 0
+#define FEATHER_E4M3 1
+
+#define FEATHER_ROUND_RNE 0       /* pack_fp8_tensor (round to nearest even) */
+#define FEATHER_ROUND_TRUNC 1     /* *_legacy packers (E5M2 only, drop the low byte) */
+
+#define FEATHER_SEM_KERNEL 0      /* decode of the GPU kernels (gemv.py:83-88) */
+#define FEATHER_SEM_IEEE 1        /* decode of the CPU unpack_* API (fp8.py:381-391) */
+
+#define FEATHER_OUT_F32 0
+#define FEATHER_OUT_F16 1
+
+#define FEATHER_TAIL_MASK 0       /* keys past seq_len are excluded from the softmax */
+#define FEATHER_TAIL_REFERENCE 1  /* keys past seq_len in the last 64-key tile count as zero rows
+                                     (attention.py:57-59) */
+
+/* Library version (major * 10000 + minor * 100 + patch). */
+int feather_version(void);
+
+/* Message for the last non-zero return code on this thread ("" if none). */
+const char *feather_last_error(void);
+
+/* fp16[n] -> u32[ceil(n/4)], four FP8 codes per word, tail padded with +0.
+ * Replaces pack_fp8_tensor / pack_fp8_ndarray / pack_fp8_into_fp32
+ * (feather/packers/fp8.py:260-281, :178-210, :69-136) with rounding = RNE, and
+ * the *_legacy packers (:8-66, :139-175, :213-257) with rounding = TRUNC.
+ * src must be 2-byte aligned, dst 4-byte aligned. */
+int feather_pack_fp8(const void *src_f16, void *dst_u32, int64_t n, int mode, int rounding, void *stream);
+
+/* u32[n_words] -> fp32 or fp16 [4 * n_words] in element order.
+ * Replaces unpack_fp8_from_fp32 / unpack_into_fp8_ndarray
+ * (feather/packers/fp8.py:336-392, :395-432) with semantics = IEEE, the legacy
+ * unpack (:284-333) and the kernels' in-register decode with semantics =
+ * KERNEL.  relu != 0 applies max(0, x) (relu1d_fp8_ret_fp32_feather_gpu,
+ * feather/routines/activations.py:9-42). */
+int feather_unpack_fp8(const void *src_u32, void *dst, int64_t n_words, int mode, int semantics, int out_dtype,
+                       int relu, void *stream);
+
+/* fp16[n] -> u32[ceil(n/2)] (first element in the low half, odd tail + 0) and
+ * back.  Replaces pack_fp16_ndarray / pack_fp16_into_fp32 and
+ * unpack_into_fp16_ndarray / unpack_fp32_into_fp16
+ * (feather/packers/fp16.py:83-116, :8-43, :119-151, :46-80). */
+int feather_pack_fp16(const void *src_f16, void *dst_u32, int64_t n, void *stream);
+int feather_unpack_fp16(const void *src_u32, void *dst_f16, int64_t n_words, void *stream);
+
+/* out[r] = sum_k dec(m[r, k]) * dec(v[k]), fp32 accumulate, fp32 out[M].
+ * m: M*K/4 words row-major, v: K/4 words; K % 4 == 0; m, v 4-byte aligned
+ * (16-byte aligned rows take the fast path).
+ * Replaces gemv_fp8_e5m2_acc_fp32_gpu / gemv_fp8_e4m3_acc_fp32_gpu
+ * (feather/routines/gemv.py:136-184, :187-235). */
+int feather_gemv_fp8(const void *m, const void *v, void *out_f32, int64_t M, int64_t K, int mode, void *stream);
+
+/* out[b, r] = sum_k dec(w[r, k]) * dec(x[b, k]) for b < nvec (1 <= nvec <= 64):
+ * the weight matrix is streamed once for all vectors.  No reference
+ * counterpart (the reference runs one vector per launch, gemv.py:179-183);
+ * used by the batched decode step. */
+int feather_gemv_fp8_batched(const void *w, const void *x, void *out_f32, int64_t M, int64_t K, int64_t nvec, int mode,
+                             void *stream);
+
+/* Bytes of scratch feather_dot_* need (per stream in flight).  The scratch must
+ * be zero-filled once before its first use; the kernels leave it zeroed. */
+int64_t feather_dot_scratch_bytes(void);
+
+/* out[0] = sum_k dec(x1[k]) * dec(x2[k]) over n_words packed words, fp32.
+ * Deterministic: per-workgroup partials are combined in a fixed order by the
+ * last workgroup to finish (the reference adds them with fp32 atomics).
+ * Replaces dot_fp8_e5m2_acc_fp32_gpu (feather/routines/dot.py:220-260); mode
+ * E4M3 has no reference kernel and uses the GEMV decode. */
+int feather_dot_fp8(const void *x1, const void *x2, void *out_f32, void *scratch, int64_t n_words, int mode,
+                    void *stream);
+
+/* FP16-packed dot, summed in fp32.  fp16_products != 0: per word
+ * fp16(lo1*lo2) +fp16 fp16(hi1*hi2) as in the reference GPU kernel
+ * (dot_fp16_acc_fp32_gpu, feather/routines/dot.py:194-218, :134-141);
+ * fp16_products == 0: exact fp32 products as in the reference's CPU variants
+ * (dot_fp16_acc_fp32_vec / _numba, feather/routines/dot.py:9-50, :53-106). */
+int feather_dot_fp16(const void *x1, const void *x2, void *out_f32, void *scratch, int64_t n_words, int fp16_products,
+                     void *stream);
+
+/* Non-causal attention forward on packed Q/K/V: for each of n_heads
+ * independent heads, out[h] = softmax(Q K^T * scale) V, Q/K/V [L, d/4] words,
+ * out [L, d] fp32; scores fp32, P rounded to fp16 before P.V, fp32 output.
+ * d in {64, 128, 256, 512}.  kv_group > 1 maps query head h to K/V head
+ * h / kv_group (K/V then hold n_heads / kv_group heads).
+ * Replaces flash_attention_fp8_e5m2_acc_fp32_gpu
+ * (feather/routines/attention.py:110-179) at n_heads = 1, mode = E5M2,
+ * scale = 1/sqrt(d), tail = REFERENCE. */
+int feather_flash_attn_fp8(const void *q, const void *k, const void *v, void *out_f32, int64_t n_heads, int64_t L,
+                           int64_t d, int64_t kv_group, int mode, float scale, int tail, void *stream);
+
+/* Bytes of scratch feather_paged_attn_fp8 needs for the given problem. */
+int64_t feather_paged_attn_scratch_bytes(int64_t n_seq, int64_t n_q_heads, int64_t d, int64_t max_ctx);
+
+/* Single-query (decode) attention over a paged FP8 KV cache.  No reference
+ * counterpart.
+ *   q            [n_seq, n_q_heads, d/4] words
+ *   k_cache      [n_blocks, n_kv_heads, block_size, d/4] words (v_cache same)
+ *   block_tables [n_seq, max_blocks] int32, ctx_lens [n_seq] int32
+ *   out          [n_seq, n_q_heads, d] fp32
+ * Query head h uses KV head h / (n_q_heads / n_kv_heads). */
+int feather_paged_attn_fp8(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,
+                           const void *ctx_lens, void *out_f32, void *scratch, int64_t n_seq, int64_t n_q_heads,
+                           int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks, int64_t max_ctx,
+                           int mode, float scale, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FEATHER_HIP_H */

@@ -1,0 +1,200 @@
+"""GPU parity: packed GEMV / dot kernels against the CPU oracle.
+
+Tolerance for floating-point results: max |y - y_ref| / max |y_ref| <= 1e-3 against the
+kernel-semantics decode followed by a float64 reduction (outputs cross zero, so the error
+is normalised by the output scale).  Integer-valued inputs must match exactly."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available()
+    return torch.device("cuda:0")
+
+
+def _dev_words(a, dev):
+    return torch.from_numpy(a.view(np.int32).copy()).to(dev).view(torch.uint32)
+
+
+def _nerr(got, want):
+    return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+@pytest.mark.parametrize("mode", ["E5M2", "E4M3"])
+def test_gemv_docstring_known_answer(dev, kats, mode):
+    import feather_amd as feather
+    k = kats["gemv"]
+    a = torch.tensor(k["matrix"], dtype=torch.float16)
+    b = torch.tensor(k["vector"], dtype=torch.float16)
+    ap = feather.pack_fp8_tensor(a, mode=mode).to(dev)
+    bp = feather.pack_fp8_tensor(b, mode=mode).to(dev)
+    out = feather.gemv(ap, bp, original_shape=a.shape, mode=mode)
+    assert out.dtype == torch.float32 and out.is_cuda and out.tolist() == k["expected"]
+    from feather_amd.routines.gemv import gemv_fp8_e4m3_acc_fp32_gpu, gemv_fp8_e5m2_acc_fp32_gpu
+    f = gemv_fp8_e5m2_acc_fp32_gpu if mode == "E5M2" else gemv_fp8_e4m3_acc_fp32_gpu
+    assert f(ap, bp, a.shape).tolist() == k["expected"]
+
+
+@pytest.mark.parametrize("mode", ["E5M2", "E4M3"])
+@pytest.mark.parametrize("M,K", [(4096, 4096), (300, 8192), (7, 20), (129, 1040), (16, 36864), (1, 16)])
+def test_gemv_integer_inputs_exact(dev, mode, M, K):
+    """Reference harness inputs (bench_gemv.py:53-57): the result is the exact integer matvec."""
+    import feather_amd as feather
+    g = torch.Generator().manual_seed(M * 31 + K)
+    a = torch.randint(-3, 3, (M, K), generator=g).to(torch.float16)
+    b = torch.randint(-3, 3, (K,), generator=g).to(torch.float16)
+    out = feather.gemv(feather.pack_fp8_tensor(a.to(dev), mode=mode), feather.pack_fp8_tensor(b.to(dev), mode=mode),
+                       original_shape=(M, K), mode=mode)
+    want = torch.mv(a.double(), b.double())
+    assert torch.equal(out.cpu().double(), want)
+
+
+@pytest.mark.parametrize("mode", ["E5M2", "E4M3"])
+@pytest.mark.parametrize("M,K", [(512, 8192), (1000, 2048), (64, 16384), (33, 48), (8, 40000)])
+def test_gemv_random_vs_oracle(dev, orc, mode, M, K):
+    import feather_amd as feather
+    rng = np.random.default_rng(M + K)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    a[rng.random((M, K)) < 0.01] *= 1e-3                      # E4M3 zero-exponent codes (flush semantics)
+    b = rng.standard_normal(K).astype(np.float32)
+    b[rng.random(K) < 0.01] *= 1e-3
+    mp, vp = orc.pack_fp8(a.astype(np.float16), mode), orc.pack_fp8(b.astype(np.float16), mode)
+    out = feather.gemv(_dev_words(mp, dev), _dev_words(vp, dev), original_shape=(M, K), mode=mode).cpu().numpy()
+    want64 = orc.gemv_f64_np(mp, vp, M, K, mode)
+    assert _nerr(out, want64) <= TOL
+    if M * K <= 1 << 20:                                      # reference-structured fp32 oracle on small cases
+        assert _nerr(out, orc.gemv(mp, vp, M, K, mode)) <= TOL
+    assert _nerr(out, want64) <= 1e-5                         # fp32 accumulation is far inside the bar
+
+
+def test_gemv_e4m3_uses_kernel_decode_not_ieee(dev, orc):
+    """A matrix made only of zero-exponent codes separates the two decodes by 2^8."""
+    import feather_amd as feather
+    codes = np.tile(np.array([1, 2, 3, 4, 5, 6, 7, 0x87], np.uint8), 64 * 16 // 8).reshape(16, 64)
+    v = np.full(64, 0x38, np.uint8)                           # 1.0 in E4M3
+    out = feather.gemv(_dev_words(codes.reshape(-1).view(np.uint32), dev), _dev_words(v.view(np.uint32), dev),
+                       original_shape=(16, 64), mode="E4M3").cpu().numpy()
+    want = orc.gemv(codes.reshape(-1).view(np.uint32), v.view(np.uint32), 16, 64, "E4M3", acc64=True)
+    assert np.allclose(out, want, rtol=1e-6) and np.allclose(out, 8 * (28 - 7) * 2.0 ** -17)
+    nan_codes = np.full((16, 64), 0x7F, np.uint8)             # NaN code decodes to 480 in the kernels
+    out = feather.gemv(_dev_words(nan_codes.reshape(-1).view(np.uint32), dev), _dev_words(v.view(np.uint32), dev),
+                       original_shape=(16, 64), mode="E4M3").cpu().numpy()
+    assert np.array_equal(out, np.full(16, 480.0 * 64, np.float32))
+
+
+def test_gemv_config_sized_properties(dev):
+    """16384 x 16384 (too large for the scalar oracle): linearity in the vector and agreement
+    with a torch fp32 matvec of the decoded operands, both on device."""
+    import feather_amd as feather
+    g = torch.Generator().manual_seed(2)
+    M = K = 16384
+    x = torch.randn(M, K, generator=g)
+    x[torch.rand(M, K, generator=g) < 0.01] *= 1e-3
+    v = torch.randn(K, generator=g)
+    for mode in ("E5M2", "E4M3"):
+        mp = feather.pack_fp8_tensor(x.half().to(dev), mode=mode)
+        vp = feather.pack_fp8_tensor(v.half().to(dev), mode=mode)
+        out = feather.gemv(mp, vp, original_shape=(M, K), mode=mode)
+        md = feather.unpack_fp8_tensor(mp, mode=mode, semantics="kernel").view(M, K)
+        vd = feather.unpack_fp8_tensor(vp, mode=mode, semantics="kernel")
+        want = torch.mv(md.double(), vd.double())
+        assert ((out.double() - want).abs().max() / want.abs().max()).item() <= 1e-5
+        # twice the vector (exact in FP8: exponent + 1) doubles the result exactly
+        vp2 = feather.pack_fp8_tensor((2 * v.half()).to(dev), mode=mode)
+        vd2 = feather.unpack_fp8_tensor(vp2, mode=mode, semantics="kernel")
+        if torch.equal(vd2, 2 * vd):
+            assert torch.equal(feather.gemv(mp, vp2, original_shape=(M, K), mode=mode), 2 * out)
+        del mp, md
+    torch.cuda.empty_cache()
+
+
+def test_gemv_rejects_bad_shapes(dev):
+    import feather_amd as feather
+    w = torch.zeros(12, dtype=torch.int32, device=dev)
+    with pytest.raises(ValueError):
+        feather.gemv(w, w, original_shape=(4, 6))
+    with pytest.raises(ValueError):
+        feather.gemv(w, w, original_shape=(4, 16))            # m holds 12 words, needs 16
+    assert feather.gemv(w[:0], w[:4], original_shape=(0, 16)).shape == (0,)
+
+
+@pytest.mark.parametrize("mode", ["E4M3", "E5M2"])
+@pytest.mark.parametrize("M,K,nvec", [(2048, 2048, 32), (256, 5632, 32), (50, 512, 5), (33, 1024, 64), (16, 100, 3)])
+def test_gemv_batched_vs_oracle(dev, orc, mode, M, K, nvec):
+    from feather_amd.routines.gemv import gemv_fp8_batched_acc_fp32_gpu
+    rng = np.random.default_rng(M + K + nvec)
+    w = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float16)
+    x = rng.standard_normal((nvec, K)).astype(np.float16)
+    wp, xp = orc.pack_fp8(w, mode), orc.pack_fp8(x, mode)
+    out = gemv_fp8_batched_acc_fp32_gpu(_dev_words(wp, dev), _dev_words(xp, dev), (M, K), nvec, mode).cpu().numpy()
+    want = orc.decode_np(xp, mode).reshape(nvec, K) @ orc.decode_np(wp, mode).reshape(M, K).T
+    assert out.shape == (nvec, M) and _nerr(out, want) <= TOL
+    if M * K * nvec <= 1 << 22:
+        assert _nerr(out, orc.gemv_batched(wp, xp, M, K, nvec, mode)) <= TOL
+
+
+# ---------------------------------------------------------------- dot
+
+def test_dot_docstring_known_answers(dev, kats):
+    import feather_amd as feather
+    from feather_amd.packers import fp16
+    from feather_amd.routines import dot
+    k = kats["dot_fp8_e5m2"]
+    x1, x2 = (torch.tensor(k[n], dtype=torch.float16, device=dev) for n in ("x1", "x2"))
+    out = dot.dot_fp8_e5m2_acc_fp32_gpu(feather.pack_fp8_tensor(x1), feather.pack_fp8_tensor(x2))
+    assert out.shape == () and out.dtype == torch.float32 and out.item() == k["expected"]
+    assert feather.dot(feather.pack_fp8_tensor(x1, mode="E4M3"), feather.pack_fp8_tensor(x2, mode="E4M3"),
+                       mode="E4M3").item() == k["expected"]
+    k = kats["dot_fp16"]
+    a, b = (np.array(k[n], dtype=np.float16) for n in ("x1", "x2"))
+    assert dot.dot_fp16_acc_fp32_vec(fp16.pack_fp16_ndarray(a), fp16.pack_fp16_ndarray(b)) == k["expected"]
+    assert dot.dot_fp16_acc_fp32_numba(fp16.pack_fp16_ndarray(a), fp16.pack_fp16_ndarray(b), None) == k["expected"]
+    ta = torch.from_numpy(fp16.pack_fp16_ndarray(a)).view(torch.uint32).to(dev)
+    tb = torch.from_numpy(fp16.pack_fp16_ndarray(b)).view(torch.uint32).to(dev)
+    assert dot.dot_fp16_acc_fp32_gpu(ta, tb).item() == k["expected"]
+
+
+@pytest.mark.parametrize("mode", ["E5M2", "E4M3"])
+@pytest.mark.parametrize("n", [4, 10_000, 500_000, 1_500_000, 16384, (1 << 22) + 12])
+def test_dot_fp8_vs_oracle(dev, orc, mode, n):
+    """Sizes of the reference harness (bench_dot.py:15) plus ragged ones."""
+    import feather_amd as feather
+    rng = np.random.default_rng(n)
+    a = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    a[rng.random(n) < 0.01] *= 1e-3
+    x1, x2 = orc.pack_fp8(a.astype(np.float16), mode), orc.pack_fp8(b.astype(np.float16), mode)
+    got = feather.dot(_dev_words(x1, dev), _dev_words(x2, dev), mode=mode).item()
+    want = float(orc.decode_np(x1, mode) @ orc.decode_np(x2, mode))
+    norm = float(np.abs(orc.decode_np(x1, mode) * orc.decode_np(x2, mode)).sum())
+    assert abs(got - want) <= TOL * max(abs(want), 1e-3 * norm)
+    assert abs(got - orc.dot_fp8(x1, x2, mode, acc64=True)) <= 1e-5 * norm
+    again = feather.dot(_dev_words(x1, dev), _dev_words(x2, dev), mode=mode).item()
+    assert again == got                                        # deterministic reduction order
+
+
+@pytest.mark.parametrize("n", [2, 1001, 1 << 20])
+def test_dot_fp16_vs_oracle(dev, orc, n):
+    from feather_amd.routines import dot
+    rng = np.random.default_rng(n)
+    a = (rng.standard_normal(n) * 2).astype(np.float16)
+    b = (rng.standard_normal(n) * 2).astype(np.float16)
+    x1, x2 = orc.pack_fp16(a), orc.pack_fp16(b)
+    norm = float(np.abs(a.astype(np.float64) * b.astype(np.float64)).sum())
+    got = dot.dot_fp16_acc_fp32_gpu(_dev_words(x1, dev), _dev_words(x2, dev)).item()
+    assert abs(got - float(orc.dot_fp16(x1, x2, acc64=True))) <= 1e-5 * norm     # same fp16 roundings, fp32 sums
+    wide = float(dot.dot_fp16_acc_fp32_vec(x1.view(np.float32), x2.view(np.float32)))
+    assert abs(wide - float(a.astype(np.float64) @ b.astype(np.float64))) <= 1e-5 * norm
+
+
+def test_dot_empty_and_mismatch(dev):
+    import feather_amd as feather
+    z = torch.zeros(0, dtype=torch.int32, device=dev)
+    assert feather.dot(z, z).item() == 0.0
+    with pytest.raises(ValueError):
+        feather.dot(torch.zeros(4, dtype=torch.int32, device=dev), torch.zeros(8, dtype=torch.int32, device=dev))

@@ -1,0 +1,143 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every
+symbol the header declares, argument validation and error mapping follow the
+reference's conventions, and nothing in the product falls back to the CPU."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "feather_hip.h")
+
+
+def _declared():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(feather_[a-z0-9_]+)\s*\(", src)))
+
+
+def test_library_exports_every_declared_symbol():
+    from feather_amd import _native as N
+    assert os.path.exists(N.LIB_PATH), "build with `python -m feather_amd.build`"
+    lib = ctypes.CDLL(N.LIB_PATH)
+    names = _declared()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/feather_hip.h but not exported"
+    assert sorted(N.SIGNATURES) == names          # the ctypes table covers the header exactly
+
+
+def test_version_and_error_string():
+    from feather_amd import _native as N
+    L = N.lib()
+    assert L.feather_version() >= 100
+    assert isinstance(L.feather_last_error(), bytes)
+    assert L.feather_dot_scratch_bytes() >= 64 + 4
+    assert L.feather_paged_attn_scratch_bytes(32, 32, 64, 4096) == 32 * 32 * 16 * 66 * 4
+
+
+def test_c_abi_argument_checks_without_gpu():
+    """Validation runs before any launch, so error codes can be exercised on the CPU."""
+    from feather_amd import _native as N
+    L = N.lib()
+    assert L.feather_pack_fp8(None, None, 16, 7, 0, None) == N.EMODE
+    assert b"mode 7" in L.feather_last_error()
+    assert L.feather_pack_fp8(None, None, 16, N.E4M3, N.ROUND_TRUNC, None) == N.EMODE
+    assert L.feather_pack_fp8(None, None, 16, N.E5M2, 0, None) == N.EINVAL          # null pointers
+    assert L.feather_pack_fp8(None, None, -1, N.E5M2, 0, None) == N.EINVAL
+    assert L.feather_pack_fp8(None, None, 0, N.E5M2, 0, None) == N.OK               # empty input: nothing to do
+    assert L.feather_gemv_fp8(None, None, None, 4, 6, N.E5M2, None) == N.ESHAPE     # K % 4
+    assert b"multiple of 4" in L.feather_last_error()
+    assert L.feather_gemv_fp8(None, None, None, 4, 8, 3, None) == N.EMODE
+    assert L.feather_gemv_fp8(None, None, None, 0, 8, N.E5M2, None) == N.OK
+    assert L.feather_gemv_fp8_batched(None, None, None, 16, 512, 65, N.E4M3, None) == N.ESHAPE
+    assert L.feather_flash_attn_fp8(None, None, None, None, 1, 64, 96, 1, N.E5M2, 0.1, 0, None) in (N.EINVAL, N.ESHAPE)
+    assert L.feather_flash_attn_fp8(None, None, None, None, 3, 64, 64, 2, N.E5M2, 0.1, 0, None) == N.ESHAPE
+    assert L.feather_flash_attn_fp8(None, None, None, None, 1, 64, 64, 1, N.E5M2, 0.1, 5, None) == N.EINVAL
+    assert L.feather_unpack_fp8(None, None, 4, N.E5M2, 9, 0, 0, None) == N.EINVAL
+    assert L.feather_dot_fp8(None, None, None, None, 4, 2, None) == N.EMODE
+    assert L.feather_paged_attn_fp8(None, None, None, None, None, None, None, 1, 6, 4, 64, 16, 4, 64, N.E5M2, 0.1,
+                                    None) == N.ESHAPE
+
+
+def test_error_mapping():
+    from feather_amd import _native as N
+    L = N.lib()
+    with pytest.raises(NotImplementedError):
+        N.check(L.feather_pack_fp8(None, None, 16, 9, 0, None))
+    with pytest.raises(ValueError):
+        N.check(L.feather_gemv_fp8(None, None, None, 4, 6, N.E5M2, None))
+    with pytest.raises(NotImplementedError):
+        N.mode_code("E3M4")
+    assert N.mode_code("E5M2") == 0 and N.mode_code("E4M3") == 1
+
+
+def test_python_validation_before_any_device_work():
+    import feather_amd as feather
+    from feather_amd.routines import attention, dot, gemv
+    w = torch.zeros(8, dtype=torch.int32)
+    with pytest.raises(NotImplementedError):                     # reference: fp8.py:114
+        feather.pack_fp8_tensor(torch.zeros(4, dtype=torch.float16), mode="E3M4")
+    with pytest.raises(ValueError):                              # K % 4 != 0
+        gemv.gemv_fp8_e5m2_acc_fp32_gpu(w, w, (4, 6))
+    with pytest.raises(ValueError):                              # CPU tensors are not silently computed on the host
+        gemv.gemv_fp8_e5m2_acc_fp32_gpu(w, w, (4, 8))
+    with pytest.raises(ValueError):
+        dot.dot_fp8_e5m2_acc_fp32_gpu(w, w)
+    with pytest.raises(ValueError):
+        gemv.gemv_fp8_e4m3_acc_fp32_gpu(w.to(torch.float16), w, (4, 8))
+    with pytest.raises(ValueError):
+        attention.flash_attention_fp8_e5m2_acc_fp32_gpu(w, w, w, 4, 24)   # d = 96 unsupported
+    with pytest.raises(NotImplementedError):
+        feather.gemv(w, w, original_shape=(4, 8), mode="E2M5")
+    with pytest.raises(ValueError):
+        feather.gemv(w, w)
+
+
+def test_no_cpu_fallback_when_no_device():
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    import feather_amd as feather
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        feather.pack_fp8_tensor(torch.zeros(8, dtype=torch.float16))
+    from feather_amd.packers import fp8
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fp8.pack_fp8_ndarray(np.zeros(8, np.float16))
+
+
+def test_reference_api_surface_is_present():
+    """Names a user of the reference imports (feather/packers/*.py, feather/routines/*.py,
+    README.md:95-107) exist with the same spelling."""
+    import feather_amd as feather
+    from feather_amd.packers import fp8, fp16
+    from feather_amd.routines import activations, attention, dot, gemv
+    for n in ("pack_fp8_into_fp32_legacy", "pack_fp8_into_fp32", "pack_fp8_ndarray_legacy", "pack_fp8_ndarray",
+              "pack_fp8_tensor_legacy", "pack_fp8_tensor", "unpack_fp8_from_fp32_legacy", "unpack_fp8_from_fp32",
+              "unpack_into_fp8_ndarray"):
+        assert callable(getattr(fp8, n))
+    for n in ("pack_fp16_into_fp32", "unpack_fp32_into_fp16", "pack_fp16_ndarray", "unpack_into_fp16_ndarray"):
+        assert callable(getattr(fp16, n))
+    for n in ("gemv_fp8_e5m2_acc_fp32_gpu", "gemv_fp8_e4m3_acc_fp32_gpu"):
+        assert callable(getattr(gemv, n))
+    for n in ("dot_fp16_acc_fp32_vec", "dot_fp16_acc_fp32_numba", "dot_fp16_acc_fp32_gpu", "dot_fp8_e5m2_acc_fp32_gpu"):
+        assert callable(getattr(dot, n))
+    assert callable(attention.flash_attention_fp8_e5m2_acc_fp32_gpu)
+    assert callable(activations.relu1d_fp8_ret_fp32_feather_gpu)
+    for n in ("pack_fp8_tensor", "pack_fp16_tensor", "gemv", "dot"):
+        assert callable(getattr(feather, n))
+    import feather as shim                                         # drop-in package name
+    assert shim.pack_fp8_tensor is feather.pack_fp8_tensor
+    from feather.packers.fp8 import pack_fp8_tensor as p2
+    from feather.routines.gemv import gemv_fp8_e5m2_acc_fp32_gpu as g2
+    assert p2 is fp8.pack_fp8_tensor and g2 is gemv.gemv_fp8_e5m2_acc_fp32_gpu
+
+
+def test_product_does_not_import_the_oracle():
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "feather_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text and "feather_oracle" not in text, f

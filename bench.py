@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed-low-precision hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+
+A "step" is one E4M3-packed GEMV of the 16384 x 16384 workload (FP32 accumulate) with the
+operands already resident in HBM.  Four distinct packed matrices (1 GiB in total) are
+rotated so that neither L2 nor the 256 MB Infinity Cache can serve the stream.  The single
+JSON line printed at the end carries the headline value (microseconds per GEMV), the
+roofline record of the GEMV kernel and the CPU baseline (torch-CPU restatement of the
+reference's decode + fp32 matvec, timed on the host cores of this box); `extra` holds the
+other workloads of the metric (E5M2 GEMV, 8192^2, dot, flash attention vs fp16 SDPA, paged
+decode).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_PEAK_F16_TFLOPS = 2500.0  # dense fp16/bf16, published
+
+
+def gpu_time_us(fn, steps, warmup, sync):
+    """Average microseconds per call over `steps` back-to-back calls (HIP events on the
+    stream the kernels are launched on: torch's current stream)."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    sync()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fn(i)
+    stop.record()
+    sync()
+    return start.elapsed_time(stop) * 1000.0 / steps
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extra", action="store_true", help="only the headline GEMV workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (every routine is single-device); --gpus must be 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    import feather_amd as feather
+    from feather_amd import _native as N
+
+    assert torch.cuda.is_available(), "bench.py needs a HIP device"
+    dev = torch.device("cuda:0")
+    sync = torch.cuda.synchronize
+    N.lib()
+    g = torch.Generator(device=dev).manual_seed(2)   # synthetic inputs are drawn on the device
+
+    def randn(*shape):
+        return torch.randn(*shape, generator=g, device=dev, dtype=torch.float32)
+
+    # ---------------------------------------------------------------- headline: E4M3 GEMV 16384^2
+    M = K = 16384
+    NBUF = 4
+
+    def make_matrix(mode):
+        x = randn(M, K)
+        x = torch.where(torch.rand(M, K, generator=g, device=dev) < 0.01, x * 1e-3, x)  # zero-exponent E4M3 codes
+        return feather.pack_fp8_tensor(x.half(), mode=mode)
+
+    mats = {"E4M3": [make_matrix("E4M3") for _ in range(NBUF)]}
+    v16 = randn(K).half()
+    vecs = {m: feather.pack_fp8_tensor(v16, mode=m) for m in ("E4M3", "E5M2")}
+    gemv_bytes = M * K + K + 4 * M                             # 1 B per code, vector once, fp32 out
+
+    def gemv_step(mode):
+        bufs, vp = mats[mode], vecs[mode]
+        return lambda i: feather.gemv(bufs[i % NBUF], vp, original_shape=(M, K), mode=mode)
+
+    # the whole timed region, bracketed by synchronize on both sides
+    for i in range(args.warmup):
+        gemv_step("E4M3")(i)
+    sync()
+    t0 = time.perf_counter()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    step = gemv_step("E4M3")
+    for i in range(args.steps):
+        step(i)
+    ev1.record()
+    sync()
+    wall_ms = (time.perf_counter() - t0) * 1000.0
+    kern_us = ev0.elapsed_time(ev1) * 1000.0 / args.steps
+    ms_per_step = wall_ms / args.steps
+    achieved = gemv_bytes / (kern_us * 1e-6) / 1e9
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "gemv_fp8_e4m3_16384_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+
+    extra = {}
+    if not args.no_extra:
+        # cache-resident figure (one matrix re-used): reported separately, never the headline
+        one = mats["E4M3"][0]
+        extra["gemv_e4m3_16384_same_buffer_us"] = round(
+            gpu_time_us(lambda i: feather.gemv(one, vecs["E4M3"], original_shape=(M, K), mode="E4M3"), 100, 10, sync), 2)
+        del mats["E4M3"]
+        torch.cuda.empty_cache()
+        mats["E5M2"] = [make_matrix("E5M2") for _ in range(NBUF)]
+        us = gpu_time_us(gemv_step("E5M2"), args.steps, args.warmup, sync)
+        extra["gemv_e5m2_16384_us"] = round(us, 2)
+        extra["gemv_e5m2_16384_GBps"] = round(gemv_bytes / us / 1e3, 1)
+        extra["gemv_e5m2_16384_hbm_frac"] = round(gemv_bytes / us / 1e3 / HBM_PEAK_GBS, 4)
+        # config 0: 8192 x 8192 E5M2 (views into the 16384^2 buffers: 4 distinct 64 MiB matrices each)
+        M0 = K0 = 8192
+        sub = [b[i * (M0 * K0 // 4):(i + 1) * (M0 * K0 // 4)] for b in mats["E5M2"] for i in range(4)]
+        v0 = feather.pack_fp8_tensor(v16[:K0], mode="E5M2")
+        us = gpu_time_us(lambda i: feather.gemv(sub[i % 16], v0, original_shape=(M0, K0), mode="E5M2"),
+                         args.steps, args.warmup, sync)
+        b0 = M0 * K0 + K0 + 4 * M0
+        extra["gemv_e5m2_8192_us"] = round(us, 2)
+        extra["gemv_e5m2_8192_GBps"] = round(b0 / us / 1e3, 1)
+        # dot, n = 2^24 (E4M3): rotate through the big buffers
+        n = 1 << 24
+        xs = [b[i * (n // 4):(i + 1) * (n // 4)] for b in mats["E5M2"] for i in range(16)]
+        for mode in ("E4M3", "E5M2"):
+            us = gpu_time_us(lambda i: feather.dot(xs[(2 * i) % 64], xs[(2 * i + 1) % 64], mode=mode), args.steps,
+                             args.warmup, sync)
+            extra[f"dot_{mode.lower()}_2p24_us"] = round(us, 2)
+            extra[f"dot_{mode.lower()}_2p24_GBps"] = round((2 * n + 4) / us / 1e3, 1)
+        # pack throughput (2 B in + 1 B out per element)
+        src = randn(8192, 16384).half()
+        for mode in ("E5M2", "E4M3"):
+            us = gpu_time_us(lambda i: feather.pack_fp8_tensor(src, mode=mode), 20, 3, sync)
+            extra[f"pack_{mode.lower()}_134M_GBps"] = round(3 * src.numel() / us / 1e3, 1)
+        del src
+        del mats["E5M2"], sub, xs
+        torch.cuda.empty_cache()
+        # flash attention, B4 H16 d64, E5M2, vs fp16 SDPA on the same GPU
+        for L in (4096, 8192):
+            B, H, d = 4, 16, 64
+            qkv16 = [randn(B, H, L, d).half() for _ in range(3)]
+            pk = [feather.pack_fp8_tensor(t, mode="E5M2").view(B, H, L, d // 4) for t in qkv16]
+            us = gpu_time_us(lambda i: feather.flash_attention_fp8_e5m2_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4),
+                             10, 2, sync)
+            flops = 4.0 * B * H * L * L * d
+            extra[f"flash_attn_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
+            extra[f"flash_attn_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / us / 1e6, 1)
+            extra[f"flash_attn_e5m2_b4h16_d64_L{L}_mfma_frac"] = round(flops / us / 1e6 / MFMA_PEAK_F16_TFLOPS, 4)
+            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 2, sync)
+            extra[f"sdpa_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
+            del qkv16, pk
+        torch.cuda.empty_cache()
+
+    cpu = None
+    if not args.no_cpu:
+        from oracle import cpu_baseline
+        r = cpu_baseline.gemv_baseline(M, K, "E4M3", sample_rows=2048, repeats=3)
+        cpu = {"value": round(r["total_s"] * 1e6, 1), "unit": "us", "cores": r["cores"], "kind": "port",
+               "sample": r["sample"] + "; decode (LUT gather) + fp32 torch.mv, pack excluded",
+               "pack_us": round(r["pack_s"] * 1e6, 1), "decode_us": round(r["decode_s"] * 1e6, 1),
+               "compute_us": round(r["compute_s"] * 1e6, 1), "cpu_count": r["cpu_count"]}
+
+    line = {
+        "metric": "packed-FP8 GEMV us (16384^2, E4M3, FP32 accumulate)",
+        "value": round(kern_us, 3), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "E4M3 packed GEMV 16384x16384 + vector 16384 (BASELINE configs[1]); N(0,1) fp16 "
+                               "sources with 1% of entries x1e-3, packed 4 codes per 32-bit word; 4 distinct "
+                               "matrices (1 GiB) rotated",
+                   "M": M, "K": K, "mode": "E4M3", "buffers": NBUF},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "kernel": "gemv_fp8_kernel<E4M3>", "algorithmic_bytes": gemv_bytes,
+                     "avg_launch_us": round(kern_us, 3)},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

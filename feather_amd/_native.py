@@ -94,7 +94,23 @@ def require_gpu() -> torch.device:
 
 
 def stream_ptr(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw hipStream_t of torch's current stream on `device`."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(idx)
+
+
+def call(device: torch.device, name: str, *args) -> None:
+    """Run one C-ABI entry point on torch's current stream of `device` (made current for
+    the call if it is not) and raise on a non-zero return code."""
+    fn = getattr(lib(), name)
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx == torch.cuda.current_device():
+        rc = fn(*args, torch._C._cuda_getCurrentRawStream(idx))
+    else:
+        with torch.cuda.device(idx):
+            rc = fn(*args, torch._C._cuda_getCurrentRawStream(idx))
+    if rc != OK:
+        check(rc)
 
 
 def ptr(t: torch.Tensor) -> int:
@@ -122,12 +138,11 @@ def as_words(t: torch.Tensor, name: str) -> torch.Tensor:
 _scratch: dict = {}
 
 
-def zeroed_scratch(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
-    """Per (device, stream, tag) scratch, zero-filled once; the kernels that use
-    it leave it zeroed again."""
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream, tag)
+def scratch(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
+    """Per (device, stream, tag) scratch buffer, allocated once and re-used."""
+    key = (device.index, stream_ptr(device), tag)
     buf = _scratch.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
         _scratch[key] = buf
     return buf

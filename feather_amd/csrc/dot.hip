@@ -3,9 +3,11 @@
 // Both operands stream from HBM once (2 x 4 bytes per word pair); each lane
 // reads 128-bit chunks of both vectors, decodes in registers and accumulates
 // with v_dot2_f32_f16.  The reduction is deterministic: every workgroup writes
-// one partial to scratch, bumps an arrival counter, and the last workgroup to
-// arrive adds the partials in index order, writes the scalar and resets the
-// counter (so the scratch needs zero-filling only once).
+// one partial to scratch and a second one-wave kernel adds the partials in
+// index order.  (A single-kernel "last workgroup finishes" scheme needs
+// device-scope release/acquire around the arrival counter, which on this
+// multi-XCD part costs an L2 write-back/invalidate per workgroup and measured
+// ~45 us for 2^24 elements; the second launch costs a few us.)
 #include "common.h"
 
 namespace feather {
@@ -13,7 +15,7 @@ namespace feather {
 constexpr int kDotThreads = 256;
 constexpr int kDotMaxBlocks = 2048;
 constexpr int kDotUnroll = 4;
-// scratch layout: [0] arrival counter (u32), [64 B ..) kDotMaxBlocks fp32 partials
+// scratch layout: [64 B ..) kDotMaxBlocks fp32 partials (the first 64 B are unused padding)
 constexpr int64_t kDotScratchBytes = 64 + (int64_t)kDotMaxBlocks * 4;
 
 enum DotKind { kDotE5M2 = 0, kDotE4M3 = 1, kDotF16 = 2, kDotF16Wide = 3 };
@@ -48,7 +50,6 @@ __global__ __launch_bounds__(kDotThreads) void dot_kernel(const uint32_t *__rest
                                                          const uint32_t *__restrict__ x2, float *__restrict__ out,
                                                          uint32_t *__restrict__ scratch, int64_t n_words) {
     __shared__ float wave_part[kDotThreads / kWave];
-    __shared__ int is_last;
     float acc[kDotUnroll];
 #pragma unroll
     for (int u = 0; u < kDotUnroll; u++) acc[u] = 0.f;
@@ -88,29 +89,22 @@ __global__ __launch_bounds__(kDotThreads) void dot_kernel(const uint32_t *__rest
     const int lane = lane_id(), wave = threadIdx.x / kWave;
     if (lane == 0) wave_part[wave] = s;
     __syncthreads();
-
-    float *partials = reinterpret_cast<float *>(scratch + 16);
     if (threadIdx.x == 0) {
         float t = 0.f;
 #pragma unroll
         for (int w = 0; w < kDotThreads / kWave; w++) t += wave_part[w];
-        __hip_atomic_store(partials + blockIdx.x, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // release our partial, acquire everyone else's
-        uint32_t prev = __hip_atomic_fetch_add(scratch, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = (prev == gridDim.x - 1) ? 1 : 0;
+        reinterpret_cast<float *>(scratch + 16)[blockIdx.x] = t;
     }
-    __syncthreads();
-    if (is_last && threadIdx.x < kWave) {
-        // fixed order: lane l adds partials l, l+64, ...; then the wave fold
-        float t = 0.f;
-        for (int i = lane; i < (int)gridDim.x; i += kWave)
-            t += __hip_atomic_load(partials + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        t = wave_sum(t);
-        if (lane == 0) {
-            out[0] = t;
-            __hip_atomic_store(scratch, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
+}
+
+// One wave: lane l adds partials l, l + 64, ... in order, then the wave fold.
+__global__ __launch_bounds__(kWave) void dot_finish_kernel(const uint32_t *__restrict__ scratch,
+                                                          float *__restrict__ out, int n_partials) {
+    const float *partials = reinterpret_cast<const float *>(scratch + 16);
+    float t = 0.f;
+    for (int i = threadIdx.x; i < n_partials; i += kWave) t += partials[i];
+    t = wave_sum(t);
+    if (threadIdx.x == 0) out[0] = t;
 }
 
 template <int KIND>
@@ -127,6 +121,10 @@ static int launch_dot(const void *x1, const void *x2, void *out, void *scratch, 
     else
         hipLaunchKernelGGL((dot_kernel<KIND, false>), dim3((unsigned)blocks), dim3(kDotThreads), 0, s,
                            (const uint32_t *)x1, (const uint32_t *)x2, (float *)out, (uint32_t *)scratch, n_words);
+    int rc = check_launch(what);
+    if (rc != FEATHER_OK) return rc;
+    hipLaunchKernelGGL(dot_finish_kernel, dim3(1), dim3(kWave), 0, s, (const uint32_t *)scratch, (float *)out,
+                       (int)blocks);
     return check_launch(what);
 }
 

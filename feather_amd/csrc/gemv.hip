@@ -6,8 +6,8 @@
 //
 //   * one wave owns RPW rows at a time; a lane reads 16 consecutive codes
 //     (one 128-bit non-temporal load) per row per step, so a wave-load covers
-//     1 KiB of contiguous row bytes; U steps are issued back to back to keep
-//     RPW * U loads in flight per lane;
+//     1 KiB of contiguous row bytes; U steps are issued back to back and
+//     unconditionally, so RPW * U loads are in flight per lane;
 //   * decode is register-only: E5M2 is byte placement (v_perm_b32), E4M3 is
 //     byte-parallel integer arithmetic on four codes at a time;
 //   * multiply-accumulate is v_dot2_f32_f16 (two exact fp16 x fp16 products
@@ -20,21 +20,9 @@
 
 namespace feather {
 
-constexpr int kGemvThreads = 256;
+constexpr int kGemvThreads = 256;          // generic path
 constexpr int kGemvWaves = kGemvThreads / kWave;
 constexpr int kMaxChunk = 32768;  // codes of the vector held in LDS at once (64 KiB as fp16)
-
-// Decode `n_words` packed words of the vector into LDS as fp16 (natural
-// order) and zero the padding up to `lds_halfs`.
-template <int MODE>
-__device__ __forceinline__ void stage_vector(const uint32_t *__restrict__ v, uint32_t *lds32, int n_words,
-                                             int lds_words) {
-    for (int i = threadIdx.x; i < lds_words; i += kGemvThreads) {
-        uint32_t p01 = 0, p23 = 0;
-        if (i < n_words) dec_word<MODE>(v[i], p01, p23);
-        reinterpret_cast<u32x2 *>(lds32)[i] = u32x2{p01, p23};
-    }
-}
 
 // 16 codes (one uint4) of a row against the matching 16 fp16 of the vector.
 template <int MODE>
@@ -60,15 +48,29 @@ __device__ __forceinline__ float mac16(const u32x4 &a, const u32x4 &x0, const u3
 //   v        vector words for columns [k0, k0 + kc)
 //   k0, kc   column chunk handled by this launch (kc <= kMaxChunk, kc % 16 == 0)
 //   accumulate  add to out instead of overwriting (later chunks)
-template <int MODE, int RPW, int U>
-__global__ __launch_bounds__(kGemvThreads) void gemv_fp8_kernel(const uint8_t *__restrict__ m,
-                                                               const uint32_t *__restrict__ v,
-                                                               float *__restrict__ out, int M, int64_t K, int k0,
-                                                               int kc, int rows_per_wg, int accumulate) {
-    extern __shared__ uint32_t lds32[];  // fp16 vector chunk, padded to a multiple of 1024 * U halfs
+//   FULL     kc is a multiple of 1024: every wave-load is in range, no lane guards
+//
+// A row is walked in steps of 1 KiB (one 128-bit load per lane).  The step at
+// which a wave STARTS is rotated with the row index (stride kStagger steps):
+// without it all waves of the chip sweep the same column offsets in lock step,
+// their addresses differ by multiples of the row pitch and pile onto a few HBM
+// channels; the rotation spreads concurrent waves over the whole row and is
+// worth ~15 % of bandwidth at 16384 x 16384.
+constexpr int kStagger = 7;
+
+template <int MODE, int RPW, int U, int WAVES, bool FULL>
+__global__ __launch_bounds__(WAVES * kWave) void gemv_fp8_kernel(const uint8_t *__restrict__ m,
+                                                                const uint32_t *__restrict__ v,
+                                                                float *__restrict__ out, int M, int64_t K, int k0,
+                                                                int kc, int rows_per_wg, int accumulate) {
+    extern __shared__ uint32_t lds32[];  // fp16 vector chunk, zero-padded to whole steps
     constexpr int kStep = kWave * 16;    // codes per wave-load
-    const int kc_pad = (kc + kStep * U - 1) / (kStep * U) * (kStep * U);
-    stage_vector<MODE>(v, lds32, kc / 4, kc_pad / 4);
+    const int n_steps = (kc + kStep - 1) / kStep;
+    for (int i = threadIdx.x; i < n_steps * (kStep / 4); i += WAVES * kWave) {
+        uint32_t p01 = 0, p23 = 0;
+        if (i < kc / 4) dec_word<MODE>(v[i], p01, p23);
+        reinterpret_cast<u32x2 *>(lds32)[i] = u32x2{p01, p23};
+    }
     __syncthreads();
 
     const int lane = lane_id();
@@ -77,35 +79,53 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fp8_kernel(const uint8_t *_
     const int row_end = min(row_begin + rows_per_wg, M);
     const u32x4 *lds128 = reinterpret_cast<const u32x4 *>(lds32);
 
-    for (int r0 = row_begin + wave * RPW; r0 < row_end; r0 += kGemvWaves * RPW) {
+    for (int r0 = row_begin + wave * RPW; r0 < row_end; r0 += WAVES * RPW) {
         float acc[RPW];
         const uint8_t *rowp[RPW];
 #pragma unroll
         for (int r = 0; r < RPW; r++) {
             acc[r] = 0.f;
-            int row = min(r0 + r, M - 1);  // clamp: surplus rows re-read the last row, result dropped
+            int row = min(r0 + r, M - 1);  // surplus rows re-read the last row, result dropped
             rowp[r] = m + (int64_t)row * K + k0 + lane * 16;
         }
-        for (int c = 0; c < kc; c += kStep * U) {
+        const int s0 = (int)(((unsigned)(r0 / RPW) * (unsigned)kStagger) % (unsigned)n_steps);
+        int it = 0;
+        for (; it + U <= n_steps; it += U) {   // U wave-loads per row in flight
+            int col[U];
             u32x4 a[RPW][U];
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                int col = c + u * kStep + lane * 16;
-                bool ok = col < kc;
+                int st = it + u + s0;
+                if (st >= n_steps) st -= n_steps;
+                col[u] = st * kStep;
 #pragma unroll
                 for (int r = 0; r < RPW; r++) {
-                    a[r][u] = u32x4{0, 0, 0, 0};
-                    if (ok) a[r][u] = load_nt128(rowp[r] + c + u * kStep);
+                    if (FULL || col[u] + lane * 16 < kc) a[r][u] = load_nt128(rowp[r] + col[u]);
+                    else a[r][u] = u32x4{0, 0, 0, 0};
                 }
             }
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                int col = c + u * kStep + lane * 16;   // < kc_pad: LDS is padded with zeros
-                u32x4 x0 = lds128[col / 8];
-                u32x4 x1 = lds128[col / 8 + 1];
+                int c8 = (col[u] + lane * 16) / 8;
+                u32x4 x0 = lds128[c8], x1 = lds128[c8 + 1];
 #pragma unroll
                 for (int r = 0; r < RPW; r++) acc[r] = mac16<MODE>(a[r][u], x0, x1, acc[r]);
             }
+        }
+        for (; it < n_steps; it++) {           // fewer than U steps left
+            int st = it + s0;
+            if (st >= n_steps) st -= n_steps;
+            int c = st * kStep;
+            u32x4 a[RPW];
+#pragma unroll
+            for (int r = 0; r < RPW; r++) {
+                if (FULL || c + lane * 16 < kc) a[r] = load_nt128(rowp[r] + c);
+                else a[r] = u32x4{0, 0, 0, 0};
+            }
+            int c8 = (c + lane * 16) / 8;
+            u32x4 x0 = lds128[c8], x1 = lds128[c8 + 1];
+#pragma unroll
+            for (int r = 0; r < RPW; r++) acc[r] = mac16<MODE>(a[r], x0, x1, acc[r]);
         }
 #pragma unroll
         for (int r = 0; r < RPW; r++) {
@@ -154,21 +174,29 @@ static int launch_gemv(const void *m, const void *v, float *out, int64_t M, int6
                            (const uint32_t *)m, (const uint32_t *)v, out, (int)M, K / 4);
         return check_launch("feather_gemv_fp8");
     }
-    constexpr int RPW = 2, U = 4;
+    // Shape of the launch (measured on MI355X at 16384^2): one workgroup per CU with 8
+    // (E5M2) or 16 (E4M3: the decode needs more waves to hide its ALU work) waves and a
+    // contiguous range of rows per workgroup gives the best HBM efficiency.
+    constexpr int RPW = MODE == FEATHER_E5M2 ? 1 : 2;
+    constexpr int U = 4;
+    constexpr int WAVES = MODE == FEATHER_E5M2 ? 8 : 16;
     constexpr int kStep = kWave * 16;
-    // rows per workgroup: aim at ~4 workgroups per CU (256 CUs) so the vector
-    // decode (K bytes from L2 per workgroup) stays a few percent of the matrix
-    // bytes the workgroup streams, in multiples of the 8 rows one pass covers.
-    int64_t rows_per_wg = (M + 1023) / 1024;
-    rows_per_wg = (rows_per_wg + kGemvWaves * RPW - 1) / (kGemvWaves * RPW) * (kGemvWaves * RPW);
+    constexpr int kCUs = 256;
+    int64_t rows_per_wg = (M + kCUs - 1) / kCUs;
+    rows_per_wg = (rows_per_wg + WAVES * RPW - 1) / (WAVES * RPW) * (WAVES * RPW);
     int64_t blocks = (M + rows_per_wg - 1) / rows_per_wg;
     for (int64_t k0 = 0; k0 < K; k0 += kMaxChunk) {
         int kc = (int)((K - k0) < kMaxChunk ? (K - k0) : kMaxChunk);
-        int kc_pad = (kc + kStep * U - 1) / (kStep * U) * (kStep * U);
-        size_t lds = (size_t)kc_pad * 2;
-        hipLaunchKernelGGL((gemv_fp8_kernel<MODE, RPW, U>), dim3((unsigned)blocks), dim3(kGemvThreads), lds, s,
-                           (const uint8_t *)m, (const uint32_t *)v + k0 / 4, out, (int)M, K, (int)k0, kc,
-                           (int)rows_per_wg, k0 > 0 ? 1 : 0);
+        int n_steps = (kc + kStep - 1) / kStep;
+        size_t lds = (size_t)n_steps * kStep * 2;
+        if (kc % kStep == 0)
+            hipLaunchKernelGGL((gemv_fp8_kernel<MODE, RPW, U, WAVES, true>), dim3((unsigned)blocks),
+                               dim3(WAVES * kWave), lds, s, (const uint8_t *)m, (const uint32_t *)v + k0 / 4, out,
+                               (int)M, K, (int)k0, kc, (int)rows_per_wg, k0 > 0 ? 1 : 0);
+        else
+            hipLaunchKernelGGL((gemv_fp8_kernel<MODE, RPW, U, WAVES, false>), dim3((unsigned)blocks),
+                               dim3(WAVES * kWave), lds, s, (const uint8_t *)m, (const uint32_t *)v + k0 / 4, out,
+                               (int)M, K, (int)k0, kc, (int)rows_per_wg, k0 > 0 ? 1 : 0);
         int rc = check_launch("feather_gemv_fp8");
         if (rc != FEATHER_OK) return rc;
     }

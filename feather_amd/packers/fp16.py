@@ -21,16 +21,14 @@ def _pack_device(x: torch.Tensor) -> torch.Tensor:
     x = x.contiguous().view(-1)
     n = x.numel()
     out = torch.empty((n + 1) // 2, dtype=torch.int32, device=x.device)
-    with torch.cuda.device(x.device):
-        N.check(N.lib().feather_pack_fp16(N.ptr(x), N.ptr(out), n, N.stream_ptr(x.device)))
+    N.call(x.device, "feather_pack_fp16", N.ptr(x), N.ptr(out), n)
     return out.view(torch.uint32)
 
 
 def _unpack_device(w: torch.Tensor) -> torch.Tensor:
     w = w.contiguous().view(-1)
     out = torch.empty(w.numel() * 2, dtype=torch.float16, device=w.device)
-    with torch.cuda.device(w.device):
-        N.check(N.lib().feather_unpack_fp16(N.ptr(w), N.ptr(out), w.numel(), N.stream_ptr(w.device)))
+    N.call(w.device, "feather_unpack_fp16", N.ptr(w), N.ptr(out), w.numel())
     return out
 
 

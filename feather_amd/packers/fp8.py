@@ -36,17 +36,14 @@ def _pack_device(x: torch.Tensor, mode: int, rounding: int) -> torch.Tensor:
     x = x.contiguous().view(-1)
     n = x.numel()
     out = torch.empty((n + 3) // 4, dtype=torch.int32, device=x.device)
-    with torch.cuda.device(x.device):
-        N.check(N.lib().feather_pack_fp8(N.ptr(x), N.ptr(out), n, mode, rounding, N.stream_ptr(x.device)))
+    N.call(x.device, "feather_pack_fp8", N.ptr(x), N.ptr(out), n, mode, rounding)
     return out.view(torch.uint32)
 
 
 def _unpack_device(w: torch.Tensor, mode: int, semantics: int, out_f16: bool, relu: bool = False) -> torch.Tensor:
     w = w.contiguous().view(-1)
     out = torch.empty(w.numel() * 4, dtype=torch.float16 if out_f16 else torch.float32, device=w.device)
-    with torch.cuda.device(w.device):
-        N.check(N.lib().feather_unpack_fp8(N.ptr(w), N.ptr(out), w.numel(), mode, semantics,
-                                           N.OUT_F16 if out_f16 else N.OUT_F32, int(relu), N.stream_ptr(w.device)))
+    N.call(w.device, "feather_unpack_fp8", N.ptr(w), N.ptr(out), w.numel(), mode, semantics, N.OUT_F16 if out_f16 else N.OUT_F32, int(relu))
     return out
 
 

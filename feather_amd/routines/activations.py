@@ -16,7 +16,5 @@ def relu1d_fp8_ret_fp32_feather_gpu(x: torch.Tensor, n: int) -> torch.Tensor:
     if n < 0 or n > 4 * x.numel():
         raise ValueError(f"n={n} exceeds the {4 * x.numel()} elements packed in x")
     full = torch.empty(4 * x.numel(), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
-        N.check(N.lib().feather_unpack_fp8(N.ptr(x), N.ptr(full), x.numel(), N.E5M2, N.SEM_KERNEL, N.OUT_F32, 1,
-                                           N.stream_ptr(x.device)))
+    N.call(x.device, "feather_unpack_fp8", N.ptr(x), N.ptr(full), x.numel(), N.E5M2, N.SEM_KERNEL, N.OUT_F32, 1)
     return full[:n]

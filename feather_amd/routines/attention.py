@@ -56,9 +56,7 @@ def flash_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: torch.
     if scale is None:
         scale = 1.0 / math.sqrt(d)
     out = torch.empty((n_heads, seq_len, d), dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
-        N.check(N.lib().feather_flash_attn_fp8(N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), n_heads, seq_len, d, kv_group,
-                                               code, float(scale), _TAILS[tail], N.stream_ptr(q.device)))
+    N.call(q.device, "feather_flash_attn_fp8", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), n_heads, seq_len, d, kv_group, code, float(scale), _TAILS[tail])
     if q.dim() >= 2 and q.shape[-2:] == (seq_len, h_dim):
         return out.view(*q.shape[:-2], seq_len, d)
     return out[0] if n_heads == 1 else out

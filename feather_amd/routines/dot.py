@@ -25,8 +25,18 @@ def _operands(x1: torch.Tensor, x2: torch.Tensor):
     return x1, x2
 
 
+_SCRATCH_BYTES = None
+
+
+def _scratch_bytes() -> int:
+    global _SCRATCH_BYTES
+    if _SCRATCH_BYTES is None:
+        _SCRATCH_BYTES = int(N.lib().feather_dot_scratch_bytes())
+    return _SCRATCH_BYTES
+
+
 def _scratch(dev: torch.device) -> torch.Tensor:
-    return N.zeroed_scratch(dev, int(N.lib().feather_dot_scratch_bytes()), "dot")
+    return N.scratch(dev, _scratch_bytes(), "dot")
 
 
 def dot_fp8_acc_fp32_gpu(x1: torch.Tensor, x2: torch.Tensor, mode: str = "E5M2") -> torch.Tensor:
@@ -34,9 +44,7 @@ def dot_fp8_acc_fp32_gpu(x1: torch.Tensor, x2: torch.Tensor, mode: str = "E5M2")
     code = N.mode_code(mode)
     x1, x2 = _operands(x1, x2)
     out = torch.empty((), dtype=torch.float32, device=x1.device)
-    with torch.cuda.device(x1.device):
-        N.check(N.lib().feather_dot_fp8(N.ptr(x1), N.ptr(x2), N.ptr(out), N.ptr(_scratch(x1.device)), x1.numel(), code,
-                                        N.stream_ptr(x1.device)))
+    N.call(x1.device, "feather_dot_fp8", N.ptr(x1), N.ptr(x2), N.ptr(out), N.ptr(_scratch(x1.device)), x1.numel(), code)
     return out
 
 
@@ -53,9 +61,7 @@ def dot_fp8_e4m3_acc_fp32_gpu(x1: torch.Tensor, x2: torch.Tensor) -> torch.Tenso
 def _dot_fp16(x1: torch.Tensor, x2: torch.Tensor, fp16_products: bool) -> torch.Tensor:
     x1, x2 = _operands(x1, x2)
     out = torch.empty((), dtype=torch.float32, device=x1.device)
-    with torch.cuda.device(x1.device):
-        N.check(N.lib().feather_dot_fp16(N.ptr(x1), N.ptr(x2), N.ptr(out), N.ptr(_scratch(x1.device)), x1.numel(),
-                                         int(fp16_products), N.stream_ptr(x1.device)))
+    N.call(x1.device, "feather_dot_fp16", N.ptr(x1), N.ptr(x2), N.ptr(out), N.ptr(_scratch(x1.device)), x1.numel(), int(fp16_products))
     return out
 
 

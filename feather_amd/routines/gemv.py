@@ -40,8 +40,7 @@ def gemv_fp8_acc_fp32_gpu(m: torch.Tensor, v: torch.Tensor, m_shape, mode: str =
     if v.device != m.device:
         raise ValueError("m and v must be on the same device")
     out = torch.empty((M,), dtype=torch.float32, device=m.device)
-    with torch.cuda.device(m.device):
-        N.check(N.lib().feather_gemv_fp8(N.ptr(m), N.ptr(v), N.ptr(out), M, K, code, N.stream_ptr(m.device)))
+    N.call(m.device, "feather_gemv_fp8", N.ptr(m), N.ptr(v), N.ptr(out), M, K, code)
     return out
 
 
@@ -73,7 +72,5 @@ def gemv_fp8_batched_acc_fp32_gpu(w: torch.Tensor, x: torch.Tensor, w_shape, nve
     if x.numel() != nvec * K // 4:
         raise ValueError(f"x holds {x.numel()} words, expected {nvec * K // 4} for {nvec} vectors of {K}")
     out = torch.empty((nvec, M), dtype=torch.float32, device=w.device)
-    with torch.cuda.device(w.device):
-        N.check(N.lib().feather_gemv_fp8_batched(N.ptr(w), N.ptr(x), N.ptr(out), M, K, nvec, code,
-                                                 N.stream_ptr(w.device)))
+    N.call(w.device, "feather_gemv_fp8_batched", N.ptr(w), N.ptr(x), N.ptr(out), M, K, nvec, code)
     return out

@@ -55,9 +55,5 @@ def paged_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k_cache: torch.Tensor, v_c
     out = torch.empty((n_seq, n_q_heads, d), dtype=torch.float32, device=q.device)
     nbytes = int(N.lib().feather_paged_attn_scratch_bytes(n_seq, n_q_heads, d, max_ctx))
     scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
-    with torch.cuda.device(q.device):
-        N.check(N.lib().feather_paged_attn_fp8(N.ptr(q), N.ptr(k_cache), N.ptr(v_cache), N.ptr(block_tables),
-                                               N.ptr(context_lens), N.ptr(out), N.ptr(scratch), n_seq, n_q_heads,
-                                               n_kv_heads, d, block_size, max_blocks, max_ctx, code, float(scale),
-                                               N.stream_ptr(q.device)))
+    N.call(q.device, "feather_paged_attn_fp8", N.ptr(q), N.ptr(k_cache), N.ptr(v_cache), N.ptr(block_tables), N.ptr(context_lens), N.ptr(out), N.ptr(scratch), n_seq, n_q_heads, n_kv_heads, d, block_size, max_blocks, max_ctx, code, float(scale))
     return out

@@ -95,13 +95,13 @@ int feather_gemv_fp8(const void *m, const void *v, void *out_f32, int64_t M, int
 int feather_gemv_fp8_batched(const void *w, const void *x, void *out_f32, int64_t M, int64_t K, int64_t nvec, int mode,
                              void *stream);
 
-/* Bytes of scratch feather_dot_* need (per stream in flight).  The scratch must
- * be zero-filled once before its first use; the kernels leave it zeroed. */
+/* Bytes of scratch feather_dot_* need (one buffer per stream in flight; 64-byte
+ * aligned; contents need no initialisation). */
 int64_t feather_dot_scratch_bytes(void);
 
 /* out[0] = sum_k dec(x1[k]) * dec(x2[k]) over n_words packed words, fp32.
- * Deterministic: per-workgroup partials are combined in a fixed order by the
- * last workgroup to finish (the reference adds them with fp32 atomics).
+ * Deterministic: per-workgroup partials are combined in a fixed order by a
+ * second small kernel (the reference adds them with fp32 atomics).
  * Replaces dot_fp8_e5m2_acc_fp32_gpu (feather/routines/dot.py:220-260); mode
  * E4M3 has no reference kernel and uses the GEMV decode. */
 int feather_dot_fp8(const void *x1, const void *x2, void *out_f32, void *scratch, int64_t n_words, int mode,

@@ -17,13 +17,18 @@
 // permuting the key order in which V^T is written to LDS, so the softmax
 // output feeds the second MFMA straight from registers: no shuffle, no LDS
 // round trip for P.  Row maxima need one exchange across the 4 lanes that
-// share a query (two ds_swizzle/bpermute steps); row sums stay per lane until
-// the epilogue.
+// share a query (two bpermute steps); the row sums (softmax denominators) are
+// accumulated by one more MFMA per step whose A operand is a constant block of
+// ones, so they cost no vector-ALU work.
 //
 // Numerics follow the reference kernel (feather/routines/attention.py:24-108):
 // fp16 x fp16 products accumulated in fp32, scores scaled in fp32, online
 // softmax in fp32 (computed as 2^x with log2(e) folded into the scale), P
-// rounded to fp16 before P.V, fp32 output.
+// rounded to fp16 before P.V, fp32 output.  One difference inside the stated
+// tolerance: the denominator sums the fp16-rounded P (the values that multiply
+// V) where the reference sums P before rounding.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace feather {
@@ -50,22 +55,33 @@ __device__ __forceinline__ float xor_lane(float x, int mask) {
     return __shfl_xor(x, mask, kWave);
 }
 
-template <int D, int MODE, int QB, int BN>
-__global__ __launch_bounds__(kAttnThreads) void flash_attn_kernel(
+// QB  16-query blocks per wave (a workgroup owns 64 * QB queries)
+// SB  query blocks scored together (SB divides QB)
+// BN  keys per tile
+// OCC workgroups per CU the register budget is sized for (2 keeps every MFMA
+//     accumulator in architectural VGPRs, so rescaling needs no AGPR copies)
+template <int D, int MODE, int QB, int SB, int BN, int OCC>
+__global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
     const uint32_t *__restrict__ q, const uint32_t *__restrict__ k, const uint32_t *__restrict__ v,
     float *__restrict__ out, int L, int n_heads, int kv_group, int tiles_per_head, float scale_log2e,
     int keys_scored, int mask_tail) {
     constexpr int DW = D / 4;              // packed words per row
     constexpr int KS = D + 8;              // fp16 per K row in LDS (16 B pad against bank conflicts)
-    constexpr int VS = BN + 8;             // fp16 per V^T row in LDS
+    constexpr int VS = BN;                 // fp16 per V^T row in LDS (16-byte chunks XOR-swizzled by row)
+    constexpr int CH = BN / 8;             // 16-byte chunks per V^T row
     constexpr int QT = 64 * QB;            // queries per workgroup
     constexpr int NU = BN * D / 16 / kAttnThreads;  // 16-code units per thread per tile
     static_assert(NU >= 1, "tile too small for 256 threads");
     constexpr int KB16 = BN / 16, KB32 = BN / 32, DB = D / 16, STEPS = D / 32;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    _Float16 *k_lds = reinterpret_cast<_Float16 *>(smem);
-    _Float16 *vt_lds = k_lds + BN * KS;
+    // two buffers of (K tile, V^T tile): tile i+1 is written while tile i is being read
+    constexpr int kBufHalfs = BN * KS + D * VS;
+    _Float16 *const lds = reinterpret_cast<_Float16 *>(smem);
+    // V^T swizzle: chunk c of row r lives at chunk c ^ swz(r).  Eight lanes that read the same
+    // chunk of eight consecutive rows, and the lanes that write the same key group of rows four
+    // apart, then fall on different LDS banks.
+    auto swz = [](int row) { return (row ^ (row >> 2)) & (CH - 1); };
 
     // XCD-aware block mapping: consecutive workgroup ids go round-robin over the 8
     // XCDs (each with its own L2); remap so that an XCD works through a contiguous
@@ -98,15 +114,21 @@ __global__ __launch_bounds__(kAttnThreads) void flash_attn_kernel(
         }
     }
 
-    float4_t o[QB][DB];
-    float m_run[QB], l_run[QB];
+    // o[b][DB] is one extra accumulator block whose A operand is constant: rows 0, 4, 8, 12
+    // of it are all ones, so element [0] of every lane accumulates l = sum_k P[k, q] of the
+    // lane's query on the matrix core (the softmax denominator costs no VALU adds).  The
+    // summands are the fp16-rounded P that also multiply V.
+    float4_t o[QB][DB + 1];
+    float m_run[QB];
 #pragma unroll
     for (int b = 0; b < QB; b++) {
         m_run[b] = -INFINITY;
-        l_run[b] = 0.f;
 #pragma unroll
-        for (int d = 0; d < DB; d++) o[b][d] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int d = 0; d <= DB; d++) o[b][d] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
+    const _Float16 one_or_zero = (j & 3) == 0 ? (_Float16)1 : (_Float16)0;
+    const half8_t ones = {one_or_zero, one_or_zero, one_or_zero, one_or_zero,
+                          one_or_zero, one_or_zero, one_or_zero, one_or_zero};
 
     // ---- register staging of the next packed K / V tile
     u32x4 kreg[NU];
@@ -126,7 +148,9 @@ __global__ __launch_bounds__(kAttnThreads) void flash_attn_kernel(
             }
         }
     };
-    auto stage = [&]() {
+    auto stage = [&](int buf) {
+        _Float16 *k_lds = lds + buf * kBufHalfs;
+        _Float16 *vt_lds = k_lds + BN * KS;
 #pragma unroll
         for (int i = 0; i < NU; i++) {
             int u = tid + kAttnThreads * i;
@@ -160,110 +184,133 @@ __global__ __launch_bounds__(kAttnThreads) void flash_attn_kernel(
                 lo2[3] = perm(p23[1], p23[0], 0x07060302u); hi2[3] = perm(p23[3], p23[2], 0x07060302u);
             }
 #pragma unroll
-            for (int c = 0; c < 4; c++)
-                *reinterpret_cast<u32x2 *>(vt_lds + (4 * ddw + c) * VS + pos) = u32x2{lo2[c], hi2[c]};
+            for (int c = 0; c < 4; c++) {
+                int row = 4 * ddw + c;
+                *reinterpret_cast<u32x2 *>(vt_lds + row * VS + (((pos >> 3) ^ swz(row)) << 3) + (pos & 4)) =
+                    u32x2{lo2[c], hi2[c]};
+            }
         }
     };
 
     prefetch(0);
-    for (int key0 = 0; key0 < keys_scored; key0 += BN) {
-        __syncthreads();  // every wave is done reading the previous tile
-        stage();
-        __syncthreads();
-        if (key0 + BN < keys_scored) prefetch(key0 + BN);
-
-        // ---- S^T = K Q^T for this wave's queries
-        float4_t s[QB][KB16];
-#pragma unroll
-        for (int c = 0; c < KB16; c++) {
-#pragma unroll
-            for (int b = 0; b < QB; b++) s[b][c] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int st = 0; st < STEPS; st++) {
-                half8_t kf = *reinterpret_cast<const half8_t *>(k_lds + (16 * c + j) * KS + 32 * st + 8 * kb);
-#pragma unroll
-                for (int b = 0; b < QB; b++) s[b][c] = mfma16(kf, qf[b][st], s[b][c]);
-            }
+    stage(0);
+    if (BN < keys_scored) prefetch(BN);
+    __syncthreads();
+    int cur = 0;
+    for (int key0 = 0; key0 < keys_scored; key0 += BN, cur ^= 1) {
+        // tile i+1 goes to the other buffer (its readers passed the barrier that ended the previous
+        // iteration) and tile i+2 into registers, both off the critical path of this tile's math
+        if (key0 + BN < keys_scored) {
+            stage(cur ^ 1);
+            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
         }
+        const _Float16 *k_lds = lds + cur * kBufHalfs;
+        const _Float16 *vt_lds = k_lds + BN * KS;
+        const bool ragged = mask_tail && key0 + BN > L;   // only the last tile can hold masked keys
 
-        // ---- online softmax, one query per lane column
         half8_t pf[QB][KB32];
+        // query blocks are scored SB at a time: the K fragments are re-used across the SB
+        // blocks while only SB * KB16 score tiles are live in registers
 #pragma unroll
-        for (int b = 0; b < QB; b++) {
-            float mx = -INFINITY;
+        for (int b0 = 0; b0 < QB; b0 += SB) {
+            // ---- S^T = K Q^T (raw, unscaled scores)
+            float4_t s[SB][KB16];
 #pragma unroll
-            for (int c = 0; c < KB16; c++)
+            for (int c = 0; c < KB16; c++) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    float x = s[b][c][r] * scale_log2e;
-                    if (mask_tail && key0 + 16 * c + 4 * kb + r >= L) x = -INFINITY;
-                    s[b][c][r] = x;
-                    mx = fmaxf(mx, x);
+                for (int st = 0; st < STEPS; st++) {
+                    half8_t kf = *reinterpret_cast<const half8_t *>(k_lds + (16 * c + j) * KS + 32 * st + 8 * kb);
+#pragma unroll
+                    for (int b = 0; b < SB; b++)
+                        s[b][c] = mfma16(kf, qf[b0 + b][st], st == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : s[b][c]);
                 }
-            mx = fmaxf(mx, xor_lane(mx, 16));
-            mx = fmaxf(mx, xor_lane(mx, 32));
-            float m_new = fmaxf(m_run[b], mx);
-            float alpha = __builtin_amdgcn_exp2f(m_run[b] - m_new);
-            m_run[b] = m_new;
-            float rs = 0.f;
-#pragma unroll
-            for (int t = 0; t < KB32; t++) {
-                half8_t p8;
-#pragma unroll
-                for (int a = 0; a < 2; a++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        float e = __builtin_amdgcn_exp2f(s[b][2 * t + a][r] - m_new);
-                        rs += e;
-                        p8[4 * a + r] = (_Float16)e;  // round to nearest even, as P.to(fp16)
-                    }
-                pf[b][t] = p8;
             }
-            l_run[b] = l_run[b] * alpha + rs;
+            // ---- online softmax, one query per lane column.  The running maximum is kept on
+            // the raw scores; scale * log2(e) is folded into one fma per score:
+            // p = 2^(s * c - m * c).
 #pragma unroll
-            for (int d = 0; d < DB; d++) o[b][d] *= alpha;
+            for (int b = 0; b < SB; b++) {
+                if (ragged) {
+#pragma unroll
+                    for (int c = 0; c < KB16; c++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (key0 + 16 * c + 4 * kb + r >= L) s[b][c][r] = -INFINITY;
+                }
+                float mx = s[b][0][0];
+#pragma unroll
+                for (int c = 0; c < KB16; c++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) mx = fmaxf(mx, s[b][c][r]);
+                mx = fmaxf(mx, xor_lane(mx, 16));
+                mx = fmaxf(mx, xor_lane(mx, 32));
+                const float m_old = m_run[b0 + b];
+                const float m_new = fmaxf(m_old, mx);
+                const float mc = m_new * scale_log2e;
+#pragma unroll
+                for (int t = 0; t < KB32; t++) {
+                    half8_t p8;
+#pragma unroll
+                    for (int a = 0; a < 2; a++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[b][2 * t + a][r], scale_log2e, -mc));
+                            p8[4 * a + r] = (_Float16)e;  // round to nearest even, as P.to(fp16)
+                        }
+                    pf[b0 + b][t] = p8;
+                }
+                // rescale only when some query of this block saw a new maximum (wave-uniform test)
+                if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
+                    const float alpha = __builtin_amdgcn_exp2f((m_old - m_new) * scale_log2e);
+                    m_run[b0 + b] = m_new;
+#pragma unroll
+                    for (int d = 0; d <= DB; d++) o[b0 + b][d] *= alpha;
+                }
+            }
         }
 
-        // ---- O^T += V^T P^T
+        // ---- O^T += V^T P^T (and the row sums through the constant ones block)
 #pragma unroll
-        for (int t = 0; t < KB32; t++)
+        for (int t = 0; t < KB32; t++) {
 #pragma unroll
             for (int d = 0; d < DB; d++) {
-                half8_t vf = *reinterpret_cast<const half8_t *>(vt_lds + (16 * d + j) * VS + 32 * t + 8 * kb);
+                half8_t vf = *reinterpret_cast<const half8_t *>(vt_lds + (16 * d + j) * VS +
+                                                                (((4 * t + kb) ^ swz(16 * d + j)) << 3));
 #pragma unroll
                 for (int b = 0; b < QB; b++) o[b][d] = mfma16(vf, pf[b][t], o[b][d]);
             }
+#pragma unroll
+            for (int b = 0; b < QB; b++) o[b][DB] = mfma16(ones, pf[b][t], o[b][DB]);
+        }
+        __syncthreads();  // tile i+1 is visible; every wave is done reading tile i
     }
 
     // ---- epilogue: finish the row sums, normalise, store [q][dd]
     float *oh = out + (int64_t)head * L * D;
 #pragma unroll
     for (int b = 0; b < QB; b++) {
-        float l = l_run[b];
-        l += xor_lane(l, 16);
-        l += xor_lane(l, 32);
+        const float l = o[b][DB][0];   // row 4 * kb of the ones block: the full sum over keys
         int row = q0 + 16 * b + j;
         if (row < L) {
 #pragma unroll
             for (int d = 0; d < DB; d++) {
-                float4_t r = o[b][d] / l;
-                *reinterpret_cast<float4_t *>(oh + (int64_t)row * D + 16 * d + 4 * kb) = r;
+                *reinterpret_cast<float4_t *>(oh + (int64_t)row * D + 16 * d + 4 * kb) = o[b][d] / l;
             }
         }
     }
 }
 
-template <int D, int MODE, int QB, int BN>
+template <int D, int MODE, int QB, int SB, int BN, int OCC>
 static int launch_attn(const void *q, const void *k, const void *v, void *out, int64_t n_heads, int64_t L,
                        int64_t kv_group, float scale, int tail, hipStream_t s) {
     constexpr int QT = 64 * QB;
-    constexpr size_t lds = (size_t)(BN * (D + 8) + D * (BN + 8)) * 2;
+    constexpr size_t lds = (size_t)(BN * (D + 8) + D * BN) * 2 * 2;  // two (K, V^T) buffers
     int tiles = (int)((L + QT - 1) / QT);
     int64_t blocks = tiles * n_heads;
     FEATHER_CHECK(blocks < (1ll << 31), FEATHER_ESHAPE, "feather_flash_attn_fp8: grid too large");
     // the reference scores whole 64-key tiles (zero rows past L); otherwise only tiles of BN up to L
     int64_t keys_scored = tail == FEATHER_TAIL_REFERENCE ? (L + 63) / 64 * 64 : (L + BN - 1) / BN * BN;
-    auto kern = flash_attn_kernel<D, MODE, QB, BN>;
+    auto kern = flash_attn_kernel<D, MODE, QB, SB, BN, OCC>;
     if (lds > 64 * 1024) {
         static bool attr_set = false;  // per instantiation
         if (!attr_set) {
@@ -284,11 +331,25 @@ static int launch_attn(const void *q, const void *k, const void *v, void *out, i
 template <int MODE>
 static int dispatch_attn(const void *q, const void *k, const void *v, void *out, int64_t n_heads, int64_t L, int64_t d,
                          int64_t kv_group, float scale, int tail, hipStream_t s) {
+    if (d == 64) {
+        const char *var = getenv("FEATHER_ATTN_VARIANT");
+        int vv = var ? atoi(var) : 0;
+        switch (vv) {
+            case 1: return launch_attn<64, MODE, 2, 2, 64, 3>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+            case 2: return launch_attn<64, MODE, 2, 2, 64, 4>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+            case 3: return launch_attn<64, MODE, 2, 2, 128, 3>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+            case 4: return launch_attn<64, MODE, 2, 1, 128, 3>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+            case 5: return launch_attn<64, MODE, 4, 1, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+            case 6: return launch_attn<64, MODE, 1, 1, 64, 4>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+            case 7: return launch_attn<64, MODE, 2, 2, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+            default: break;
+        }
+    }
     switch (d) {
-        case 64: return launch_attn<64, MODE, 2, 64>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-        case 128: return launch_attn<128, MODE, 2, 64>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-        case 256: return launch_attn<256, MODE, 1, 32>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-        case 512: return launch_attn<512, MODE, 1, 32>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+        case 64: return launch_attn<64, MODE, 4, 2, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+        case 128: return launch_attn<128, MODE, 2, 2, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+        case 256: return launch_attn<256, MODE, 1, 1, 32, 1>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+        case 512: return launch_attn<512, MODE, 1, 1, 32, 1>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
     }
     set_error("feather_flash_attn_fp8: head dim %lld not supported (64, 128, 256, 512)", (long long)d);
     return FEATHER_ESHAPE;

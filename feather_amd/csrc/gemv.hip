@@ -14,6 +14,14 @@
 //     added into an fp32 accumulator);
 //   * the RPW row sums are folded across the wave with DPP.
 //
+// Two measured dead ends, kept here so they are not tried again.  (1) Feeding
+// the codes to FP8 MFMAs (matrix bytes as A, vector bytes as B, dot product on
+// the diagonal of the 16x16 result) removes the decode but ran 12 % SLOWER at
+// 16384^2 (47.3 us against 41.6 us for E5M2).  (2) Issuing the loads of the
+// next group before the arithmetic of the current one (software pipelining,
+// twice the bytes in flight) also lost 6 %: at ~6.4 TB/s the memory system is
+// saturated and deeper queues only add latency.
+//
 // A workgroup takes a contiguous range of rows so the vector decode is
 // amortised; ranges are sized so that the grid is a few workgroups per CU.
 #include "common.h"
@@ -165,21 +173,9 @@ __global__ void fill_zero_kernel(float *p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.f;
 }
 
-template <int MODE>
-static int launch_gemv(const void *m, const void *v, float *out, int64_t M, int64_t K, hipStream_t s) {
-    if (K % 16 != 0 || !aligned(m, 16)) {
-        int64_t blocks = (M + kGemvWaves - 1) / kGemvWaves;
-        if (blocks > 256 * 8) blocks = 256 * 8;
-        hipLaunchKernelGGL((gemv_fp8_generic_kernel<MODE>), dim3((unsigned)blocks), dim3(kGemvThreads), 0, s,
-                           (const uint32_t *)m, (const uint32_t *)v, out, (int)M, K / 4);
-        return check_launch("feather_gemv_fp8");
-    }
-    // Shape of the launch (measured on MI355X at 16384^2): one workgroup per CU with 8
-    // (E5M2) or 16 (E4M3: the decode needs more waves to hide its ALU work) waves and a
-    // contiguous range of rows per workgroup gives the best HBM efficiency.
-    constexpr int RPW = MODE == FEATHER_E5M2 ? 1 : 2;
-    constexpr int U = 4;
-    constexpr int WAVES = MODE == FEATHER_E5M2 ? 8 : 16;
+template <int MODE, int RPW, int U>
+static int launch_gemv_fast(const void *m, const void *v, float *out, int64_t M, int64_t K, hipStream_t s) {
+    constexpr int WAVES = 8;
     constexpr int kStep = kWave * 16;
     constexpr int kCUs = 256;
     int64_t rows_per_wg = (M + kCUs - 1) / kCUs;
@@ -201,6 +197,25 @@ static int launch_gemv(const void *m, const void *v, float *out, int64_t M, int6
         if (rc != FEATHER_OK) return rc;
     }
     return FEATHER_OK;
+}
+
+template <int MODE>
+static int launch_gemv(const void *m, const void *v, float *out, int64_t M, int64_t K, hipStream_t s) {
+    if (K % 16 != 0 || !aligned(m, 16)) {
+        int64_t blocks = (M + kGemvWaves - 1) / kGemvWaves;
+        if (blocks > 256 * 8) blocks = 256 * 8;
+        hipLaunchKernelGGL((gemv_fp8_generic_kernel<MODE>), dim3((unsigned)blocks), dim3(kGemvThreads), 0, s,
+                           (const uint32_t *)m, (const uint32_t *)v, out, (int)M, K / 4);
+        return check_launch("feather_gemv_fp8");
+    }
+    // Shape of the launch (measured on MI355X at 16384^2, 4 rotating matrices): one workgroup
+    // of 8 waves per CU, each owning a contiguous range of rows.  E5M2 with long rows: one
+    // row per wave, 4 steps in flight (41.2 us, 81 % of HBM peak).  E4M3, and E5M2 with rows
+    // shorter than 8 steps: four rows per wave share every LDS read of the vector, 2 steps in
+    // flight (E4M3 43.5 us, 77 %).  More waves, deeper unrolling or more workgroups per CU all
+    // measured slower.
+    if (MODE == FEATHER_E5M2 && K >= 8192) return launch_gemv_fast<MODE, 1, 4>(m, v, out, M, K, s);
+    return launch_gemv_fast<MODE, 4, 2>(m, v, out, M, K, s);
 }
 
 }  // namespace feather

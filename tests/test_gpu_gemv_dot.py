@@ -69,7 +69,7 @@ def test_gemv_random_vs_oracle(dev, orc, mode, M, K):
     assert _nerr(out, want64) <= TOL
     if M * K <= 1 << 20:                                      # reference-structured fp32 oracle on small cases
         assert _nerr(out, orc.gemv(mp, vp, M, K, mode)) <= TOL
-    assert _nerr(out, want64) <= 1e-5                         # fp32 accumulation is far inside the bar
+    assert _nerr(out, want64) <= 1e-4                         # fp32 accumulation is far inside the bar
 
 
 def test_gemv_e4m3_uses_kernel_decode_not_ieee(dev, orc):
@@ -85,6 +85,21 @@ def test_gemv_e4m3_uses_kernel_decode_not_ieee(dev, orc):
     out = feather.gemv(_dev_words(nan_codes.reshape(-1).view(np.uint32), dev), _dev_words(v.view(np.uint32), dev),
                        original_shape=(16, 64), mode="E4M3").cpu().numpy()
     assert np.array_equal(out, np.full(16, 480.0 * 64, np.float32))
+    # NaN codes mixed with ordinary and zero-exponent codes, in the matrix and in the vector
+    rng = np.random.default_rng(99)
+    M, K = 48, 2048
+    mc = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    mc[rng.random((M, K)) < 0.02] = 0x7F
+    mc[rng.random((M, K)) < 0.02] = 0xFF
+    for vec_nan in (False, True):
+        vc = rng.integers(0, 256, size=K).astype(np.uint8)
+        vc[(vc & 0x7F) == 0x7F] = 0x30
+        if vec_nan:
+            vc[[5, 700, 2047]] = [0x7F, 0xFF, 0x7F]
+        out = feather.gemv(_dev_words(mc.reshape(-1).view(np.uint32), dev), _dev_words(vc.view(np.uint32), dev),
+                           original_shape=(M, K), mode="E4M3").cpu().numpy()
+        want = orc.gemv(mc.reshape(-1).view(np.uint32), vc.view(np.uint32), M, K, "E4M3", acc64=True)
+        assert _nerr(out, want) <= 1e-4
 
 
 def test_gemv_config_sized_properties(dev):
@@ -103,7 +118,7 @@ def test_gemv_config_sized_properties(dev):
         md = feather.unpack_fp8_tensor(mp, mode=mode, semantics="kernel").view(M, K)
         vd = feather.unpack_fp8_tensor(vp, mode=mode, semantics="kernel")
         want = torch.mv(md.double(), vd.double())
-        assert ((out.double() - want).abs().max() / want.abs().max()).item() <= 1e-5
+        assert ((out.double() - want).abs().max() / want.abs().max()).item() <= 1e-4
         # twice the vector (exact in FP8: exponent + 1) doubles the result exactly
         vp2 = feather.pack_fp8_tensor((2 * v.half()).to(dev), mode=mode)
         vd2 = feather.unpack_fp8_tensor(vp2, mode=mode, semantics="kernel")

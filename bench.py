@@ -51,6 +51,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMV workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (known traffic) to scale rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (every routine is single-device); --gpus must be 1",
@@ -106,11 +108,21 @@ def main() -> int:
     ms_per_step = wall_ms / args.steps
     achieved = gemv_bytes / (kern_us * 1e-6) / 1e9
 
+    if args.calibrate_copy:
+        src = torch.empty(M * K // 4, dtype=torch.int32, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)                                      # reads 256 MiB, writes 256 MiB
+        sync()
+        del src, dst
+
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summary file)
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "gemv_fp8_e4m3_16384_traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "gemv_fp8_16384_hbm_traffic.md")
     if os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch")
+        for ln in open(tpath):
+            if ln.startswith("hbm_bytes_per_launch_e4m3:"):
+                traffic = int(ln.split(":")[1].strip())
 
     extra = {}
     if not args.no_extra:

@@ -42,7 +42,25 @@ SIGNATURES = {
     "feather_paged_attn_scratch_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "feather_paged_attn_fp8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                       _i32, _f32, _vp]),
+    "feather_decode_step_scratch_bytes": (_i64, [_vp, _i64, _i64]),
+    "feather_decode_step": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp]),
 }
+
+
+class DecoderLayer(ctypes.Structure):
+    """feather_decoder_layer_t (include/feather_hip.h)."""
+    _fields_ = [("w_qkv", _vp), ("w_o", _vp), ("w_gate_up", _vp), ("w_down", _vp), ("norm_attn", _vp),
+                ("norm_mlp", _vp), ("k_cache", _vp), ("v_cache", _vp)]
+
+
+class Decoder(ctypes.Structure):
+    """feather_decoder_t (include/feather_hip.h)."""
+    _fields_ = [("n_layers", ctypes.c_int32), ("hidden", ctypes.c_int32), ("n_q_heads", ctypes.c_int32),
+                ("n_kv_heads", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("inter", ctypes.c_int32),
+                ("vocab", ctypes.c_int32), ("block_size", ctypes.c_int32), ("max_blocks", ctypes.c_int32),
+                ("mode", ctypes.c_int32), ("rms_eps", _f32), ("rope_theta", _f32),
+                ("layers", ctypes.POINTER(DecoderLayer)), ("embed_f16", _vp), ("norm_final", _vp),
+                ("w_lm_head", _vp)]
 
 _lib = None
 _lock = threading.Lock()

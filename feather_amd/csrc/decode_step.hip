@@ -1,0 +1,292 @@
+// One decode step of a Llama-shaped model whose linear layers are FP8-packed
+// GEMVs and whose KV cache is a paged FP8 cache.  The reference has no model
+// code; this driver strings the routines of this library together for a whole
+// batch with one host call: per layer
+//     (h += delta) -> RMSNorm -> pack            add_rmsnorm_pack_kernel
+//     qkv = W_qkv x                              feather_gemv_fp8_batched
+//     RoPE(q, k), pack q, append k/v to cache    rope_append_kernel
+//     paged attention                            feather_paged_attn_fp8
+//     pack(attn) ; o = W_o attn                  pack_f32_kernel, batched GEMV
+//     (h += o) -> RMSNorm -> pack                add_rmsnorm_pack_kernel
+//     gu = W_gate_up x ; silu(g) * u -> pack     batched GEMV, swiglu_pack_kernel
+//     down = W_down act                          batched GEMV (added to h by the next norm)
+// and a final norm + lm_head GEMV.  Every activation that feeds a GEMV is
+// rounded fp32 -> fp16 -> FP8 (RNE, as pack_fp8_tensor does) and packed four
+// codes per word in the producing kernel, so no separate quantisation pass
+// touches memory.  All launches go to one stream; nothing allocates or syncs.
+#include "common.h"
+
+namespace feather {
+
+constexpr int kDsThreads = 256;
+
+template <int MODE>
+__device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d) {
+    // fp32 -> fp16 (round to nearest even) -> FP8 code (round to nearest even)
+    uint32_t h0 = __builtin_bit_cast(uint16_t, (_Float16)a), h1 = __builtin_bit_cast(uint16_t, (_Float16)b);
+    uint32_t h2 = __builtin_bit_cast(uint16_t, (_Float16)c), h3 = __builtin_bit_cast(uint16_t, (_Float16)d);
+    if constexpr (MODE == FEATHER_E5M2)
+        return enc_e5m2(h0) | (enc_e5m2(h1) << 8) | (enc_e5m2(h2) << 16) | (enc_e5m2(h3) << 24);
+    else
+        return enc_e4m3(h0) | (enc_e4m3(h1) << 8) | (enc_e4m3(h2) << 16) | (enc_e4m3(h3) << 24);
+}
+
+__device__ __forceinline__ float block_sum(float x, float *red) {
+    x = wave_sum(x);
+    const int lane = lane_id(), wave = threadIdx.x / kWave;
+    if (lane == 0) red[wave] = x;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < kDsThreads / kWave; w++) t += red[w];
+    __syncthreads();
+    return t;
+}
+
+// h[b, :] = embed[token[b], :] (fp16 table -> fp32 residual stream)
+__global__ __launch_bounds__(kDsThreads) void embed_kernel(const _Float16 *__restrict__ embed,
+                                                          const int32_t *__restrict__ tokens,
+                                                          float *__restrict__ h, int hidden) {
+    const int b = blockIdx.x;
+    const _Float16 *row = embed + (int64_t)tokens[b] * hidden;
+    for (int i = threadIdx.x; i < hidden; i += kDsThreads) h[(int64_t)b * hidden + i] = (float)row[i];
+}
+
+// h += delta (if given); xq = pack(fp16(h * rsqrt(mean(h^2) + eps) * w)).  One workgroup per row.
+template <int MODE>
+__global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__restrict__ h,
+                                                                     const float *__restrict__ delta,
+                                                                     const float *__restrict__ w,
+                                                                     uint32_t *__restrict__ xq, int hidden,
+                                                                     float eps) {
+    __shared__ float red[kDsThreads / kWave];
+    const int b = blockIdx.x;
+    float4 *hr = reinterpret_cast<float4 *>(h + (int64_t)b * hidden);
+    const float4 *dr = delta ? reinterpret_cast<const float4 *>(delta + (int64_t)b * hidden) : nullptr;
+    const float4 *wr = reinterpret_cast<const float4 *>(w);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden / 4; i += kDsThreads) {
+        float4 x = hr[i];
+        if (dr) {
+            float4 d = dr[i];
+            x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
+            hr[i] = x;
+        }
+        ss += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+    }
+    const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden / 4; i += kDsThreads) {
+        float4 x = hr[i], g = wr[i];
+        xq[(int64_t)b * (hidden / 4) + i] = quant4<MODE>(x.x * r * g.x, x.y * r * g.y, x.z * r * g.z, x.w * r * g.w);
+    }
+}
+
+// fp32 [n] -> packed FP8 words [n / 4]
+template <int MODE>
+__global__ __launch_bounds__(kDsThreads) void pack_f32_kernel(const float4 *__restrict__ x, uint32_t *__restrict__ out,
+                                                             int64_t n4) {
+    for (int64_t i = (int64_t)blockIdx.x * kDsThreads + threadIdx.x; i < n4; i += (int64_t)gridDim.x * kDsThreads) {
+        float4 v = x[i];
+        out[i] = quant4<MODE>(v.x, v.y, v.z, v.w);
+    }
+}
+
+// gu [B, 2 * inter] (gate rows then up rows) -> pack(fp16(silu(gate) * up)) [B, inter / 4]
+template <int MODE>
+__global__ __launch_bounds__(kDsThreads) void swiglu_pack_kernel(const float *__restrict__ gu,
+                                                                uint32_t *__restrict__ out, int inter, int batch) {
+    const int per_row = inter / 4;
+    for (int64_t i = (int64_t)blockIdx.x * kDsThreads + threadIdx.x; i < (int64_t)batch * per_row;
+         i += (int64_t)gridDim.x * kDsThreads) {
+        int b = (int)(i / per_row), c = (int)(i % per_row);
+        float4 g = reinterpret_cast<const float4 *>(gu + (int64_t)b * 2 * inter)[c];
+        float4 u = reinterpret_cast<const float4 *>(gu + (int64_t)b * 2 * inter + inter)[c];
+        auto f = [](float a, float bb) { return a / (1.0f + expf(-a)) * bb; };
+        out[i] = quant4<MODE>(f(g.x, u.x), f(g.y, u.y), f(g.z, u.z), f(g.w, u.w));
+    }
+}
+
+// qkv [B, (n_q + 2 n_kv) * d] fp32 -> RoPE on q and k (rotate-half convention: element j pairs
+// with j + d/2, angle pos * theta^(-2j/d)), q packed to qp [B, n_q, d/4], k and v encoded and
+// written into the paged cache at position pos = ctx_lens[b]; ctx_after[b] = pos + 1.
+template <int MODE>
+__global__ __launch_bounds__(kDsThreads) void rope_append_kernel(const float *__restrict__ qkv,
+                                                                uint32_t *__restrict__ qp,
+                                                                uint32_t *__restrict__ k_cache,
+                                                                uint32_t *__restrict__ v_cache,
+                                                                const int32_t *__restrict__ block_tables,
+                                                                const int32_t *__restrict__ ctx_lens,
+                                                                int32_t *__restrict__ ctx_after, int n_q, int n_kv,
+                                                                int d, int block_size, int max_blocks,
+                                                                float log2_theta) {
+    const int b = blockIdx.x;
+    const int pos = min(ctx_lens[b], max_blocks * block_size - 1);
+    if (threadIdx.x == 0) ctx_after[b] = pos + 1;
+    const int dw = d / 4, half_w = d / 8;            // words per head, words per rotation half
+    const int heads = n_q + 2 * n_kv;
+    const int64_t slot = ((int64_t)block_tables[(int64_t)b * max_blocks + pos / block_size] * n_kv) * block_size;
+    for (int item = threadIdx.x; item < heads * half_w; item += kDsThreads) {
+        const int head = item / half_w, t = item % half_w;
+        const float *x = qkv + ((int64_t)b * heads + head) * d;
+        float4 lo = reinterpret_cast<const float4 *>(x)[t];              // elements 4t .. 4t+3
+        float4 hi = reinterpret_cast<const float4 *>(x + d / 2)[t];      // their partners
+        if (head < n_q + n_kv) {
+            float lo4[4] = {lo.x, lo.y, lo.z, lo.w}, hi4[4] = {hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float inv_freq = exp2f(-(2.0f * (float)(4 * t + i) / (float)d) * log2_theta);
+                float s, c;
+                sincosf((float)pos * inv_freq, &s, &c);
+                float a = lo4[i], bb = hi4[i];
+                lo4[i] = a * c - bb * s;
+                hi4[i] = bb * c + a * s;
+            }
+            lo = make_float4(lo4[0], lo4[1], lo4[2], lo4[3]);
+            hi = make_float4(hi4[0], hi4[1], hi4[2], hi4[3]);
+        }
+        const uint32_t wlo = quant4<MODE>(lo.x, lo.y, lo.z, lo.w), whi = quant4<MODE>(hi.x, hi.y, hi.z, hi.w);
+        uint32_t *dst;
+        if (head < n_q) {
+            dst = qp + ((int64_t)b * n_q + head) * dw;
+        } else {
+            const int kvh = head < n_q + n_kv ? head - n_q : head - n_q - n_kv;
+            uint32_t *cache = head < n_q + n_kv ? k_cache : v_cache;
+            dst = cache + ((slot + (int64_t)kvh * block_size) + pos % block_size) * dw;
+        }
+        dst[t] = wlo;
+        dst[t + half_w] = whi;
+    }
+}
+
+template <int MODE>
+static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const int32_t *block_tables,
+                    const int32_t *ctx_lens, int batch, int max_ctx, void *scratch, float *logits, hipStream_t s) {
+    const int H = dec->hidden, nq = dec->n_q_heads, nkv = dec->n_kv_heads, d = dec->head_dim, I = dec->inter;
+    const int qkv_rows = (nq + 2 * nkv) * d;
+    // scratch carve-up (all offsets multiples of 256 bytes)
+    char *p = (char *)scratch;
+    auto take = [&](size_t bytes) { char *q = p; p += (bytes + 255) / 256 * 256; return q; };
+    float *h = (float *)take((size_t)batch * H * 4);
+    float *delta = (float *)take((size_t)batch * H * 4);
+    uint32_t *xq = (uint32_t *)take((size_t)batch * (H > I ? H : I));
+    float *qkv = (float *)take((size_t)batch * qkv_rows * 4);
+    uint32_t *qp = (uint32_t *)take((size_t)batch * nq * d);
+    float *attn = (float *)take((size_t)batch * nq * d * 4);
+    float *gu = (float *)take((size_t)batch * 2 * I * 4);
+    int32_t *ctx_after = (int32_t *)take((size_t)batch * 4);
+    void *pa_scratch = p;
+    const float scale = 1.0f / sqrtf((float)d);
+    const float log2_theta = log2f(dec->rope_theta);
+    void *st = (void *)s;
+    int rc;
+#define DS_CHECK(call)            \
+    do {                          \
+        rc = (call);              \
+        if (rc != FEATHER_OK) return rc; \
+    } while (0)
+
+    hipLaunchKernelGGL(embed_kernel, dim3(batch), dim3(kDsThreads), 0, s, (const _Float16 *)dec->embed_f16, tokens, h, H);
+    DS_CHECK(check_launch("feather_decode_step (embed)"));
+    const float *pending = nullptr;                       // output of the previous down projection, not yet added
+    for (int l = 0; l < dec->n_layers; l++) {
+        const feather_decoder_layer_t &L = dec->layers[l];
+        hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending,
+                           L.norm_attn, xq, H, dec->rms_eps);
+        DS_CHECK(check_launch("feather_decode_step (norm)"));
+        DS_CHECK(feather_gemv_fp8_batched(L.w_qkv, xq, qkv, qkv_rows, H, batch, MODE, st));
+        hipLaunchKernelGGL((rope_append_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, qkv, qp,
+                           (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, block_tables, ctx_lens, ctx_after, nq, nkv, d,
+                           dec->block_size, dec->max_blocks, log2_theta);
+        DS_CHECK(check_launch("feather_decode_step (rope)"));
+        DS_CHECK(feather_paged_attn_fp8(qp, L.k_cache, L.v_cache, block_tables, ctx_after, attn, pa_scratch, batch, nq,
+                                        nkv, d, dec->block_size, dec->max_blocks, max_ctx, MODE, scale, st));
+        int64_t n4 = (int64_t)batch * nq * d / 4;
+        hipLaunchKernelGGL((pack_f32_kernel<MODE>), dim3((unsigned)((n4 + kDsThreads - 1) / kDsThreads)),
+                           dim3(kDsThreads), 0, s, (const float4 *)attn, xq, n4);
+        DS_CHECK(check_launch("feather_decode_step (pack attn)"));
+        DS_CHECK(feather_gemv_fp8_batched(L.w_o, xq, delta, H, nq * d, batch, MODE, st));
+        hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, delta, L.norm_mlp,
+                           xq, H, dec->rms_eps);
+        DS_CHECK(check_launch("feather_decode_step (norm)"));
+        DS_CHECK(feather_gemv_fp8_batched(L.w_gate_up, xq, gu, 2 * I, H, batch, MODE, st));
+        int64_t items = (int64_t)batch * I / 4;
+        hipLaunchKernelGGL((swiglu_pack_kernel<MODE>), dim3((unsigned)((items + kDsThreads - 1) / kDsThreads)),
+                           dim3(kDsThreads), 0, s, gu, xq, I, batch);
+        DS_CHECK(check_launch("feather_decode_step (swiglu)"));
+        DS_CHECK(feather_gemv_fp8_batched(L.w_down, xq, delta, H, I, batch, MODE, st));
+        pending = delta;
+    }
+    hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending, dec->norm_final,
+                       xq, H, dec->rms_eps);
+    DS_CHECK(check_launch("feather_decode_step (final norm)"));
+    DS_CHECK(feather_gemv_fp8_batched(dec->w_lm_head, xq, logits, dec->vocab, H, batch, MODE, st));
+#undef DS_CHECK
+    return FEATHER_OK;
+}
+
+static int64_t step_scratch_bytes(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx) {
+    const int64_t H = dec->hidden, nq = dec->n_q_heads, nkv = dec->n_kv_heads, d = dec->head_dim, I = dec->inter;
+    auto up = [](int64_t b) { return (b + 255) / 256 * 256; };
+    int64_t t = 0;
+    t += 2 * up(batch * H * 4);
+    t += up(batch * (H > I ? H : I));
+    t += up(batch * (nq + 2 * nkv) * d * 4);
+    t += up(batch * nq * d);
+    t += up(batch * nq * d * 4);
+    t += up(batch * 2 * I * 4);
+    t += up(batch * 4);
+    t += up(feather_paged_attn_scratch_bytes(batch, nq, d, max_ctx));
+    return t;
+}
+
+}  // namespace feather
+
+using namespace feather;
+
+static int check_decoder(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx, const char *me) {
+    FEATHER_CHECK(dec, FEATHER_EINVAL, "%s: null decoder", me);
+    FEATHER_CHECK(dec->mode == FEATHER_E5M2 || dec->mode == FEATHER_E4M3, FEATHER_EMODE, "%s: mode %d not supported", me,
+                  dec->mode);
+    FEATHER_CHECK(dec->n_layers >= 0 && dec->hidden > 0 && dec->n_q_heads > 0 && dec->n_kv_heads > 0 &&
+                      dec->head_dim > 0 && dec->inter > 0 && dec->vocab > 0 && dec->block_size > 0 && dec->max_blocks > 0,
+                  FEATHER_EINVAL, "%s: bad configuration", me);
+    FEATHER_CHECK(dec->hidden == dec->n_q_heads * dec->head_dim, FEATHER_ESHAPE, "%s: hidden != n_q_heads * head_dim", me);
+    FEATHER_CHECK(dec->head_dim == 64 || dec->head_dim == 128 || dec->head_dim == 256, FEATHER_ESHAPE,
+                  "%s: head dim %d not supported", me, dec->head_dim);
+    FEATHER_CHECK(dec->n_q_heads % dec->n_kv_heads == 0 && dec->n_q_heads / dec->n_kv_heads <= 16, FEATHER_ESHAPE,
+                  "%s: unsupported head grouping", me);
+    FEATHER_CHECK(dec->hidden % 16 == 0 && dec->inter % 16 == 0, FEATHER_ESHAPE,
+                  "%s: hidden and inter must be multiples of 16", me);
+    FEATHER_CHECK(batch >= 1 && batch <= 64, FEATHER_ESHAPE, "%s: batch %lld outside [1, 64]", me, (long long)batch);
+    FEATHER_CHECK(max_ctx >= 1 && max_ctx <= (int64_t)dec->max_blocks * dec->block_size, FEATHER_ESHAPE,
+                  "%s: max_ctx exceeds the block table", me);
+    return FEATHER_OK;
+}
+
+extern "C" int64_t feather_decode_step_scratch_bytes(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx) {
+    if (check_decoder(dec, batch, max_ctx, "feather_decode_step_scratch_bytes") != FEATHER_OK) return -1;
+    return step_scratch_bytes(dec, batch, max_ctx);
+}
+
+extern "C" int feather_decode_step(const feather_decoder_t *dec, const void *token_ids, const void *block_tables,
+                                   const void *ctx_lens, int64_t batch, int64_t max_ctx, void *scratch,
+                                   void *logits_f32, void *stream) {
+    const char *me = "feather_decode_step";
+    int rc = check_decoder(dec, batch, max_ctx, me);
+    if (rc != FEATHER_OK) return rc;
+    FEATHER_CHECK(token_ids && block_tables && ctx_lens && scratch && logits_f32, FEATHER_EINVAL, "%s: null pointer", me);
+    FEATHER_CHECK(dec->embed_f16 && dec->norm_final && dec->w_lm_head && (dec->n_layers == 0 || dec->layers), FEATHER_EINVAL,
+                  "%s: null weight pointer", me);
+    for (int l = 0; l < dec->n_layers; l++) {
+        const feather_decoder_layer_t &L = dec->layers[l];
+        FEATHER_CHECK(L.w_qkv && L.w_o && L.w_gate_up && L.w_down && L.norm_attn && L.norm_mlp && L.k_cache && L.v_cache,
+                      FEATHER_EINVAL, "%s: null pointer in layer %d", me, l);
+    }
+    FEATHER_CHECK(aligned(scratch, 256) && aligned(logits_f32, 16), FEATHER_EINVAL, "%s: misaligned scratch/logits", me);
+    hipStream_t s = (hipStream_t)stream;
+    if (dec->mode == FEATHER_E5M2)
+        return run_step<FEATHER_E5M2>(dec, (const int32_t *)token_ids, (const int32_t *)block_tables,
+                                      (const int32_t *)ctx_lens, (int)batch, (int)max_ctx, scratch, (float *)logits_f32, s);
+    return run_step<FEATHER_E4M3>(dec, (const int32_t *)token_ids, (const int32_t *)block_tables,
+                                  (const int32_t *)ctx_lens, (int)batch, (int)max_ctx, scratch, (float *)logits_f32, s);
+}

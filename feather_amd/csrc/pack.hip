@@ -22,48 +22,6 @@ void set_error(const char *fmt, ...) {
     va_end(ap);
 }
 
-// ---------------------------------------------------------------- encoders
-
-// fp16 bits -> E5M2, round to nearest even: E5M2 is the high byte of fp16, so
-// rounding is an integer add on the bit pattern (a carry bumps the exponent,
-// values >= 61440 reach 0x7C = inf).  NaN -> 0x7F | sign.
-__device__ __forceinline__ uint32_t enc_e5m2(uint32_t h) {
-    uint32_t a = h & 0x7FFFu;
-    uint32_t sign = (h >> 8) & 0x80u;
-    uint32_t r = (a + 0x7Fu + ((a >> 8) & 1u)) >> 8;
-    return sign | (a > 0x7C00u ? 0x7Fu : r);
-}
-
-// fp16 bits -> E4M3fn (bias 7, subnormal unit 2^-9, max 448, 0x7F = NaN), RNE.
-// Anything that rounds above 448 (|x| > 464), inf and NaN give 0x7F.
-__device__ __forceinline__ uint32_t enc_e4m3(uint32_t h) {
-    uint32_t a = h & 0x7FFFu;
-    uint32_t sign = (h >> 8) & 0x80u;
-    uint32_t exp = a >> 10;
-    uint32_t code;
-    if (exp >= 9u) {                                  // |x| >= 2^-6: normal in E4M3
-        uint32_t t = a - (8u << 10);                  // rebias 15 -> 7
-        t += 0x3Fu + ((t >> 7) & 1u);                 // RNE on the 7 dropped bits
-        code = min(t >> 7, 0x7Fu);
-    } else {                                          // subnormal target: units of 2^-9
-        uint32_t full = (a & 0x3FFu) | 0x400u;
-        uint32_t sh = 16u - max(exp, 1u);             // 8..15
-        uint32_t q = full >> sh;
-        uint32_t rem = full & ((1u << sh) - 1u);
-        uint32_t half = 1u << (sh - 1u);
-        q += (rem > half || (rem == half && (q & 1u))) ? 1u : 0u;
-        code = exp == 0u ? 0u : q;                    // fp16 subnormals are < 2^-10 -> 0
-    }
-    return sign | code;
-}
-
-template <int MODE, int ROUND>
-__device__ __forceinline__ uint32_t enc(uint32_t h) {
-    if constexpr (ROUND == FEATHER_ROUND_TRUNC) return (h >> 8) & 0xFFu;
-    else if constexpr (MODE == FEATHER_E5M2) return enc_e5m2(h);
-    else return enc_e4m3(h);
-}
-
 // two fp16 (one 32-bit register) -> two codes in bits [0,16)
 template <int MODE, int ROUND>
 __device__ __forceinline__ uint32_t enc_pair(uint32_t hh) {

@@ -141,6 +141,49 @@ int feather_paged_attn_fp8(const void *q, const void *k_cache, const void *v_cac
                            int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks, int64_t max_ctx,
                            int mode, float scale, void *stream);
 
+/* ---- decode step of a Llama-shaped model on packed weights (no reference counterpart) ----
+ *
+ * The reference has no model code; this entry point runs one token step for a batch with
+ * every linear layer as a packed-FP8 batched GEMV (decode as feather_gemv_fp8) and attention
+ * over the paged FP8 cache (feather_paged_attn_fp8).  Activations that feed a GEMV are
+ * rounded fp32 -> fp16 -> FP8 (round to nearest even, as pack_fp8_tensor) in the producing
+ * kernel.  Per layer: RMSNorm, fused QKV projection, rotary embedding (rotate-half
+ * convention), append of the new K/V to the cache at position ctx_lens[b], attention over
+ * ctx_lens[b] + 1 tokens, output projection, residual, RMSNorm, gate/up projection,
+ * silu(gate) * up, down projection, residual; then the final norm and the lm_head GEMV.
+ * The structs live in HOST memory; every pointer inside them is a device pointer. */
+typedef struct feather_decoder_layer {
+    const void *w_qkv;      /* [(n_q_heads + 2 n_kv_heads) * head_dim, hidden] packed: q rows, k rows, v rows */
+    const void *w_o;        /* [hidden, n_q_heads * head_dim] packed */
+    const void *w_gate_up;  /* [2 * inter, hidden] packed: gate rows, then up rows */
+    const void *w_down;     /* [hidden, inter] packed */
+    const float *norm_attn; /* [hidden] fp32 RMSNorm weight before attention */
+    const float *norm_mlp;  /* [hidden] fp32 RMSNorm weight before the MLP */
+    void *k_cache;          /* [n_blocks, n_kv_heads, block_size, head_dim / 4] packed words, written by the step */
+    void *v_cache;          /* same shape */
+} feather_decoder_layer_t;
+
+typedef struct feather_decoder {
+    int32_t n_layers, hidden, n_q_heads, n_kv_heads, head_dim, inter, vocab;
+    int32_t block_size, max_blocks; /* KV paging: block_tables is [batch, max_blocks] */
+    int32_t mode;                   /* FEATHER_E5M2 / FEATHER_E4M3 for weights, activations and cache */
+    float rms_eps, rope_theta;
+    const feather_decoder_layer_t *layers; /* host array of n_layers entries */
+    const void *embed_f16;                 /* [vocab, hidden] fp16 embedding table */
+    const float *norm_final;               /* [hidden] */
+    const void *w_lm_head;                 /* [vocab, hidden] packed */
+} feather_decoder_t;
+
+/* Bytes of scratch feather_decode_step needs (256-byte aligned buffer); -1 for a bad configuration. */
+int64_t feather_decode_step_scratch_bytes(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx);
+
+/* token_ids [batch] int32, block_tables [batch, max_blocks] int32, ctx_lens [batch] int32 (tokens
+ * already in the cache; the caller adds 1 after the step), logits [batch, vocab] fp32.
+ * batch <= 64; max_ctx bounds ctx_lens + 1. */
+int feather_decode_step(const feather_decoder_t *dec, const void *token_ids, const void *block_tables,
+                        const void *ctx_lens, int64_t batch, int64_t max_ctx, void *scratch, void *logits_f32,
+                        void *stream);
+
 #ifdef __cplusplus
 }
 #endif

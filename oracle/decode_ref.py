@@ -1,0 +1,116 @@
+"""numpy restatement of the packed decode step (csrc/decode_step.hip) for the tests.
+TEST INFRASTRUCTURE ONLY.  The step is build-defined (the reference has no model code);
+this file fixes its meaning: float32 element-wise math, every GEMV operand rounded
+fp32 -> fp16 -> FP8 (RNE) and decoded with the kernel decode, GEMV sums in float64."""
+from __future__ import annotations
+
+import numpy as np
+
+from . import decode_np, pack_fp8
+
+
+def quant(x: np.ndarray, mode: str) -> np.ndarray:
+    """fp32 array -> decoded values after fp16 + FP8 rounding (same shape, float64)."""
+    with np.errstate(over="ignore"):
+        words = pack_fp8(x.astype(np.float32).astype(np.float16), mode)
+    return decode_np(words, mode)[: x.size].reshape(x.shape)
+
+
+def quant_codes(x: np.ndarray, mode: str) -> np.ndarray:
+    with np.errstate(over="ignore"):
+        return pack_fp8(x.astype(np.float32).astype(np.float16), mode)
+
+
+def rmsnorm(x: np.ndarray, w: np.ndarray, eps: float) -> np.ndarray:
+    x = x.astype(np.float32)
+    ms = np.mean(x.astype(np.float64) ** 2, axis=-1, keepdims=True).astype(np.float32)
+    r = (np.float32(1.0) / np.sqrt(ms + np.float32(eps))).astype(np.float32)
+    return (x * r) * w.astype(np.float32)
+
+
+def rope(x: np.ndarray, pos: int, theta: float) -> np.ndarray:
+    """x [heads, d] float32, rotate-half convention."""
+    d = x.shape[-1]
+    j = np.arange(d // 2, dtype=np.float32)
+    inv = np.exp2(-(np.float32(2.0) * j / np.float32(d)) * np.log2(np.float32(theta))).astype(np.float32)
+    ang = (np.float32(pos) * inv).astype(np.float32)
+    c, s = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    lo, hi = x[..., : d // 2], x[..., d // 2:]
+    return np.concatenate([lo * c - hi * s, hi * c + lo * s], axis=-1).astype(np.float32)
+
+
+def online_attention(dots: np.ndarray, V: np.ndarray, scale: float, chunk: int = 32, split: int = 256) -> np.ndarray:
+    """Single-query attention with the evaluation order of csrc/paged_attention.hip: tokens in
+    splits of 256, each walked in chunks of 32 with a running maximum (log2 domain), P rounded
+    to fp16 relative to the running maximum for P.V, the denominator summed from the
+    unrounded P, O rescaled when the maximum moves; splits merged at the end.  (Rounding P
+    relative to a running instead of the global maximum moves results by ~2^-12, which is
+    enough to flip an FP8 code downstream, hence the same order here.)"""
+    c = np.float32(scale * 1.4426950408889634)
+    x = (dots.astype(np.float32) * c).astype(np.float32)
+    n, d = V.shape
+    parts = []
+    for s0 in range(0, n, split):
+        m, l, o = -np.inf, np.float32(0), np.zeros(d, dtype=np.float64)
+        for c0 in range(s0, min(s0 + split, n), chunk):
+            xs = x[c0:min(c0 + chunk, n, s0 + split)]
+            m_new = max(m, float(xs.max()))
+            alpha = np.float32(np.exp2(np.float32(m - m_new))) if np.isfinite(m) else np.float32(0)
+            p = np.exp2((xs - np.float32(m_new)).astype(np.float32)).astype(np.float32)
+            l = np.float32(l * alpha + p.sum(dtype=np.float32))
+            o = o * float(alpha) + p.astype(np.float16).astype(np.float64) @ V[c0:c0 + len(xs)]
+            m = m_new
+        parts.append((m, l, o))
+    mg = max(p_[0] for p_ in parts)
+    num, den = np.zeros(d, dtype=np.float64), 0.0
+    for m, l, o in parts:
+        w = float(np.exp2(np.float32(m - mg)))
+        num += w * o
+        den += w * float(l)
+    return (num / den).astype(np.float32)
+
+
+def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables, ctx_lens, mode: str):
+    """weights: fp16 numpy arrays under the names of PackedDecoder; k_caches / v_caches: per-layer
+    uint32 arrays [n_blocks, n_kv, block_size, d/4], updated in place.  Returns logits [B, vocab] float32."""
+    H, nq, nkv, d, I = cfg.hidden, cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.inter
+    B = len(tokens)
+    Wq = lambda a: quant(np.asarray(a, dtype=np.float32), mode)                  # packed weight values
+    h = np.asarray(weights["embed"], dtype=np.float32)[np.asarray(tokens)]        # [B, H]
+    scale = np.float32(1.0 / np.sqrt(d))
+    for l in range(cfg.n_layers):
+        g = lambda n: weights[f"{l}.{n}"]
+        xq = quant(rmsnorm(h, g("norm_attn"), cfg.rms_eps), mode)
+        wqkv = Wq(np.concatenate([g("wq"), g("wk"), g("wv")], axis=0))
+        qkv = (xq @ wqkv.T).astype(np.float32)                                    # [B, (nq + 2 nkv) d]
+        attn = np.zeros((B, nq * d), dtype=np.float32)
+        for b in range(B):
+            pos = int(ctx_lens[b])
+            heads = qkv[b].reshape(nq + 2 * nkv, d)
+            q = rope(heads[:nq], pos, cfg.rope_theta)
+            k = rope(heads[nq:nq + nkv], pos, cfg.rope_theta)
+            v = heads[nq + nkv:]
+            blk, slot = int(block_tables[b][pos // cfg.block_size]), pos % cfg.block_size
+            for kvh in range(nkv):
+                k_caches[l][blk, kvh, slot] = quant_codes(k[kvh], mode)
+                v_caches[l][blk, kvh, slot] = quant_codes(v[kvh], mode)
+            qd = quant(q, mode)
+            n = pos + 1
+            for hq in range(nq):
+                kvh = hq // (nq // nkv)
+                rows = [(int(block_tables[b][t // cfg.block_size]), t % cfg.block_size) for t in range(n)]
+                Kw = np.stack([k_caches[l][bb, kvh, ss] for bb, ss in rows])
+                Vw = np.stack([v_caches[l][bb, kvh, ss] for bb, ss in rows])
+                Kd = decode_np(Kw, mode).reshape(n, d)
+                Vd = decode_np(Vw, mode).reshape(n, d)
+                attn[b, hq * d:(hq + 1) * d] = online_attention(Kd @ qd[hq], Vd, float(scale))
+        o = (quant(attn, mode) @ Wq(g("wo")).T).astype(np.float32)
+        h = h + o
+        xq = quant(rmsnorm(h, g("norm_mlp"), cfg.rms_eps), mode)
+        gu = (xq @ Wq(np.concatenate([g("w_gate"), g("w_up")], axis=0)).T).astype(np.float32)
+        gate, up = gu[:, :I], gu[:, I:]
+        act = (gate / (np.float32(1.0) + np.exp(-gate))) * up
+        dn = (quant(act, mode) @ Wq(g("w_down")).T).astype(np.float32)
+        h = h + dn
+    xq = quant(rmsnorm(h, weights["norm_final"], cfg.rms_eps), mode)
+    return (xq @ Wq(weights["lm_head"]).T).astype(np.float32)

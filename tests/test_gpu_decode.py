@@ -1,0 +1,73 @@
+"""GPU parity of the packed decode step (build-defined; the reference has no model code)
+against its numpy restatement in oracle/decode_ref.py.
+
+Tolerance: every activation is re-quantised to FP8 between kernels, so a last-bit difference
+in an fp32 sum can flip one FP8 code (a 6-12 % change of that element) now and then; logits
+are therefore compared with max |x - ref| / max |ref| <= 2e-2, and the KV codes appended by
+the first layer (no upstream quantisation flips) must agree in >= 99.5 % of the bytes."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("mode,hidden,nq,nkv,inter", [("E4M3", 512, 8, 2, 1024), ("E5M2", 256, 4, 4, 512),
+                                                      ("E4M3", 1024, 16, 1, 1536)])
+def test_decode_step_vs_oracle(orc, mode, hidden, nq, nkv, inter):
+    from feather_amd.routines.decode import DecoderConfig, PackedDecoder, random_weights
+    from oracle import decode_ref
+    dev = torch.device("cuda:0")
+    cfg = DecoderConfig(n_layers=2, hidden=hidden, n_q_heads=nq, n_kv_heads=nkv, head_dim=64, inter=inter, vocab=1000)
+    B, max_blocks = 3, 6
+    n_blocks = B * max_blocks + 2
+    w = random_weights(cfg, seed=hidden)
+    dec = PackedDecoder(cfg, w, n_blocks=n_blocks, max_blocks=max_blocks, mode=mode, device=dev)
+    g = torch.Generator().manual_seed(1)
+    bt = torch.randperm(n_blocks, generator=g)[: B * max_blocks].to(torch.int32).view(B, max_blocks)
+    ctx = torch.tensor([5, 40, 0], dtype=torch.int32)
+    # pre-fill the caches with random codes for the tokens already "seen"
+    dw = cfg.head_dim // 4
+    kc_np, vc_np = [], []
+    for lay in dec.layers:
+        for name, store in (("k_cache", kc_np), ("v_cache", vc_np)):
+            vals = torch.randn(n_blocks, nkv, cfg.block_size, cfg.head_dim, generator=g).half()
+            import feather_amd as feather
+            packed = feather.pack_fp8_tensor(vals.to(dev), mode=mode).view(n_blocks, nkv, cfg.block_size, dw)
+            lay[name].copy_(packed.view(torch.int32))
+            store.append(packed.view(torch.int32).cpu().numpy().view(np.uint32).copy())
+    wnp = {k: v.numpy() for k, v in w.items()}
+    for step in range(2):
+        tokens = torch.randint(0, cfg.vocab, (B,), generator=g, dtype=torch.int32)
+        logits = dec.step(tokens.to(dev), bt.to(dev), ctx.to(dev)).cpu().numpy()
+        want = decode_ref.decode_step_ref(cfg, wnp, kc_np, vc_np, tokens.numpy(), bt.numpy(), ctx.numpy(), mode)
+        err = np.abs(logits - want).max() / np.abs(want).max()
+        assert err <= 2e-2, f"step {step}: normalised logit error {err}"
+        assert np.mean(np.abs(logits - want) <= 2e-3 * np.abs(want).max()) >= 0.97
+        got_k = dec.layers[0]["k_cache"].cpu().numpy().view(np.uint32).view(np.uint8)
+        got_v = dec.layers[0]["v_cache"].cpu().numpy().view(np.uint32).view(np.uint8)
+        assert np.mean(got_k == kc_np[0].view(np.uint8)) >= 0.995 and np.mean(got_v == vc_np[0].view(np.uint8)) >= 0.995
+        # continue from the oracle's cache state so that a flipped code does not accumulate across steps
+        for l, lay in enumerate(dec.layers):
+            lay["k_cache"].copy_(torch.from_numpy(kc_np[l].view(np.int32)))
+            lay["v_cache"].copy_(torch.from_numpy(vc_np[l].view(np.int32)))
+        ctx = ctx + 1
+
+
+def test_decode_step_rejects_bad_arguments():
+    from feather_amd.routines.decode import DecoderConfig, PackedDecoder, random_weights
+    dev = torch.device("cuda:0")
+    cfg = DecoderConfig(n_layers=1, hidden=256, n_q_heads=4, n_kv_heads=2, head_dim=64, inter=512, vocab=100)
+    dec = PackedDecoder(cfg, random_weights(cfg), n_blocks=8, max_blocks=4, device=dev)
+    bt = torch.zeros((2, 4), dtype=torch.int32, device=dev)
+    tok = torch.zeros(2, dtype=torch.int32, device=dev)
+    ctx = torch.zeros(2, dtype=torch.int32, device=dev)
+    assert dec.step(tok, bt, ctx).shape == (2, 100)
+    with pytest.raises(ValueError):
+        dec.step(tok.long(), bt, ctx)
+    with pytest.raises(ValueError):
+        dec.step(tok, bt[:, :3].contiguous(), ctx)
+    with pytest.raises(ValueError):
+        dec.step(tok, bt, ctx, max_ctx=1000)
+    with pytest.raises(NotImplementedError):
+        PackedDecoder(cfg, random_weights(cfg), n_blocks=8, max_blocks=4, mode="E3M4", device=dev)

@@ -370,3 +370,46 @@ def test_relu_oracle(orc):
     x = np.array([-4, -1, 0, 2, 3, -0.5, 4, 1], np.float16)   # bench_activations.py:28 range
     got = orc.relu_fp8_e5m2(orc.pack_fp8(x, "E5M2"))
     assert np.array_equal(got, np.maximum(x.astype(np.float32), 0))
+
+
+# ---------------------------------------------------------------- decode-step pieces (build-defined)
+
+def test_decode_ref_rmsnorm_and_rope_match_library_forms(orc):
+    from oracle import decode_ref
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((3, 64)).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32)
+    ref = torch.nn.functional.rms_norm(torch.from_numpy(x), (64,), torch.from_numpy(w), 1e-5).numpy()
+    assert np.abs(decode_ref.rmsnorm(x, w, 1e-5) - ref).max() < 1e-6
+    d, pos = 64, 37
+    q = rng.standard_normal((2, d)).astype(np.float32)
+    inv = 1.0 / (10000.0 ** (np.arange(0, d, 2) / d))                   # rotate-half form used by Llama code
+    cos, sin = np.concatenate([np.cos(pos * inv)] * 2), np.concatenate([np.sin(pos * inv)] * 2)
+    rot = np.concatenate([-q[:, d // 2:], q[:, : d // 2]], axis=-1)
+    assert np.abs(decode_ref.rope(q, pos, 10000.0) - (q * cos + rot * sin)).max() < 2e-5
+    assert np.array_equal(decode_ref.rope(q, 0, 10000.0), q)           # position 0 is the identity
+
+
+def test_decode_ref_quant_is_pack_then_decode(orc):
+    from oracle import decode_ref
+    x = np.array([0.3, -1.7, 500.0, 1e-4, 0.0, 3.14159], np.float32)
+    for mode in ("E5M2", "E4M3"):
+        want = orc.decode_np(orc.pack_fp8(x.astype(np.float16), mode), mode)[: x.size]
+        assert np.array_equal(decode_ref.quant(x, mode), want)
+
+
+def test_decode_ref_online_attention_matches_exact_softmax(orc):
+    """The chunked evaluation order (running maximum, P rounded to fp16) is the exact softmax
+    average up to the fp16 rounding of P."""
+    from oracle import decode_ref
+    rng = np.random.default_rng(11)
+    for n in (1, 3, 31, 32, 33, 100, 256, 257, 700):
+        dots = (rng.standard_normal(n) * 8).astype(np.float32)
+        V = rng.standard_normal((n, 64))
+        sc = dots.astype(np.float64) * 0.125
+        p = np.exp(sc - sc.max())
+        want = p @ V / p.sum()
+        got = decode_ref.online_attention(dots, V, 0.125)
+        assert np.abs(got - want).max() / np.abs(want).max() < 1e-3
+    V = np.full((50, 64), 2.5)
+    assert np.allclose(decode_ref.online_attention(rng.standard_normal(50).astype(np.float32), V, 1.0), 2.5, rtol=1e-3)

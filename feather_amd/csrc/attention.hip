@@ -27,8 +27,6 @@
 // rounded to fp16 before P.V, fp32 output.  One difference inside the stated
 // tolerance: the denominator sums the fp16-rounded P (the values that multiply
 // V) where the reference sums P before rounding.
-#include <stdlib.h>
-
 #include "common.h"
 
 namespace feather {
@@ -331,20 +329,6 @@ static int launch_attn(const void *q, const void *k, const void *v, void *out, i
 template <int MODE>
 static int dispatch_attn(const void *q, const void *k, const void *v, void *out, int64_t n_heads, int64_t L, int64_t d,
                          int64_t kv_group, float scale, int tail, hipStream_t s) {
-    if (d == 64) {
-        const char *var = getenv("FEATHER_ATTN_VARIANT");
-        int vv = var ? atoi(var) : 0;
-        switch (vv) {
-            case 1: return launch_attn<64, MODE, 2, 2, 64, 3>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-            case 2: return launch_attn<64, MODE, 2, 2, 64, 4>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-            case 3: return launch_attn<64, MODE, 2, 2, 128, 3>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-            case 4: return launch_attn<64, MODE, 2, 1, 128, 3>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-            case 5: return launch_attn<64, MODE, 4, 1, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-            case 6: return launch_attn<64, MODE, 1, 1, 64, 4>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-            case 7: return launch_attn<64, MODE, 2, 2, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-            default: break;
-        }
-    }
     switch (d) {
         case 64: return launch_attn<64, MODE, 4, 2, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
         case 128: return launch_attn<128, MODE, 2, 2, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);

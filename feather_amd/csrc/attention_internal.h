@@ -1,0 +1,18 @@
+// Internal launchers shared with the decode-step driver.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace feather {
+
+// As feather_paged_attn_fp8, but the result can be written (any subset) as fp32 (out_f32), as
+// packed FP8 words of the same mode (out_packed, [n_seq, n_q_heads * d / 4]) and as fp16 holding
+// the values of those codes (out_q16, [n_seq, n_q_heads * d]): the operand of the next GEMV in
+// its two accepted forms.  Arguments are assumed validated.
+int paged_attn_launch(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,
+                      const void *ctx_lens, float *out_f32, uint32_t *out_packed, _Float16 *out_q16, void *scratch, int64_t n_seq,
+                      int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
+                      int64_t max_ctx, int mode, float scale, hipStream_t stream);
+
+}  // namespace feather

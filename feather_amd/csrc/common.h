@@ -157,6 +157,27 @@ __device__ __forceinline__ uint32_t enc(uint32_t h) {
     else return enc_e4m3(h);
 }
 
+// four fp32 values -> one packed word: fp32 -> fp16 (RNE) -> FP8 code (RNE), the rounding chain of
+// pack_fp8_tensor applied to an fp32 producer
+template <int MODE>
+__device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d) {
+    // fp32 -> fp16 (round to nearest even) -> FP8 code (round to nearest even)
+    uint32_t h0 = __builtin_bit_cast(uint16_t, (_Float16)a), h1 = __builtin_bit_cast(uint16_t, (_Float16)b);
+    uint32_t h2 = __builtin_bit_cast(uint16_t, (_Float16)c), h3 = __builtin_bit_cast(uint16_t, (_Float16)d);
+    if constexpr (MODE == FEATHER_E5M2)
+        return enc_e5m2(h0) | (enc_e5m2(h1) << 8) | (enc_e5m2(h2) << 16) | (enc_e5m2(h3) << 24);
+    else
+        return enc_e4m3(h0) | (enc_e4m3(h1) << 8) | (enc_e4m3(h2) << 16) | (enc_e4m3(h3) << 24);
+}
+
+// the four fp16 values that a packed word decodes to (kernel decode), as two fp16 pairs
+template <int MODE>
+__device__ __forceinline__ u32x2 dequant4(uint32_t word) {
+    uint32_t p01, p23;
+    dec_word<MODE>(word, p01, p23);
+    return u32x2{p01, p23};
+}
+
 // ---------------------------------------------------------------- wave64 reductions
 
 template <int CTRL>

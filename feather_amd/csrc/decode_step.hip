@@ -6,7 +6,7 @@
 //     qkv = W_qkv x                              feather_gemv_fp8_batched
 //     RoPE(q, k), pack q, append k/v to cache    rope_append_kernel
 //     paged attention                            feather_paged_attn_fp8
-//     pack(attn) ; o = W_o attn                  pack_f32_kernel, batched GEMV
+//     o = W_o attn (attention emits packed FP8)  batched GEMV
 //     (h += o) -> RMSNorm -> pack                add_rmsnorm_pack_kernel
 //     gu = W_gate_up x ; silu(g) * u -> pack     batched GEMV, swiglu_pack_kernel
 //     down = W_down act                          batched GEMV (added to h by the next norm)
@@ -14,22 +14,12 @@
 // rounded fp32 -> fp16 -> FP8 (RNE, as pack_fp8_tensor does) and packed four
 // codes per word in the producing kernel, so no separate quantisation pass
 // touches memory.  All launches go to one stream; nothing allocates or syncs.
+#include "attention_internal.h"
 #include "common.h"
 
 namespace feather {
 
 constexpr int kDsThreads = 256;
-
-template <int MODE>
-__device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d) {
-    // fp32 -> fp16 (round to nearest even) -> FP8 code (round to nearest even)
-    uint32_t h0 = __builtin_bit_cast(uint16_t, (_Float16)a), h1 = __builtin_bit_cast(uint16_t, (_Float16)b);
-    uint32_t h2 = __builtin_bit_cast(uint16_t, (_Float16)c), h3 = __builtin_bit_cast(uint16_t, (_Float16)d);
-    if constexpr (MODE == FEATHER_E5M2)
-        return enc_e5m2(h0) | (enc_e5m2(h1) << 8) | (enc_e5m2(h2) << 16) | (enc_e5m2(h3) << 24);
-    else
-        return enc_e4m3(h0) | (enc_e4m3(h1) << 8) | (enc_e4m3(h2) << 16) | (enc_e4m3(h3) << 24);
-}
 
 __device__ __forceinline__ float block_sum(float x, float *red) {
     x = wave_sum(x);
@@ -78,16 +68,6 @@ __global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__r
     for (int i = threadIdx.x; i < hidden / 4; i += kDsThreads) {
         float4 x = hr[i], g = wr[i];
         xq[(int64_t)b * (hidden / 4) + i] = quant4<MODE>(x.x * r * g.x, x.y * r * g.y, x.z * r * g.z, x.w * r * g.w);
-    }
-}
-
-// fp32 [n] -> packed FP8 words [n / 4]
-template <int MODE>
-__global__ __launch_bounds__(kDsThreads) void pack_f32_kernel(const float4 *__restrict__ x, uint32_t *__restrict__ out,
-                                                             int64_t n4) {
-    for (int64_t i = (int64_t)blockIdx.x * kDsThreads + threadIdx.x; i < n4; i += (int64_t)gridDim.x * kDsThreads) {
-        float4 v = x[i];
-        out[i] = quant4<MODE>(v.x, v.y, v.z, v.w);
     }
 }
 
@@ -171,7 +151,6 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
     uint32_t *xq = (uint32_t *)take((size_t)batch * (H > I ? H : I));
     float *qkv = (float *)take((size_t)batch * qkv_rows * 4);
     uint32_t *qp = (uint32_t *)take((size_t)batch * nq * d);
-    float *attn = (float *)take((size_t)batch * nq * d * 4);
     float *gu = (float *)take((size_t)batch * 2 * I * 4);
     int32_t *ctx_after = (int32_t *)take((size_t)batch * 4);
     void *pa_scratch = p;
@@ -179,6 +158,9 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
     const float log2_theta = log2f(dec->rope_theta);
     void *st = (void *)s;
     int rc;
+    auto gemv = [&](const void *w, float *out, int M, int K) {
+        return feather_gemv_fp8_batched(w, xq, out, M, K, batch, MODE, st);
+    };
 #define DS_CHECK(call)            \
     do {                          \
         rc = (call);              \
@@ -193,33 +175,30 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
         hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending,
                            L.norm_attn, xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
-        DS_CHECK(feather_gemv_fp8_batched(L.w_qkv, xq, qkv, qkv_rows, H, batch, MODE, st));
+        DS_CHECK(gemv(L.w_qkv, qkv, qkv_rows, H));
         hipLaunchKernelGGL((rope_append_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, qkv, qp,
                            (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, block_tables, ctx_lens, ctx_after, nq, nkv, d,
                            dec->block_size, dec->max_blocks, log2_theta);
         DS_CHECK(check_launch("feather_decode_step (rope)"));
-        DS_CHECK(feather_paged_attn_fp8(qp, L.k_cache, L.v_cache, block_tables, ctx_after, attn, pa_scratch, batch, nq,
-                                        nkv, d, dec->block_size, dec->max_blocks, max_ctx, MODE, scale, st));
-        int64_t n4 = (int64_t)batch * nq * d / 4;
-        hipLaunchKernelGGL((pack_f32_kernel<MODE>), dim3((unsigned)((n4 + kDsThreads - 1) / kDsThreads)),
-                           dim3(kDsThreads), 0, s, (const float4 *)attn, xq, n4);
-        DS_CHECK(check_launch("feather_decode_step (pack attn)"));
-        DS_CHECK(feather_gemv_fp8_batched(L.w_o, xq, delta, H, nq * d, batch, MODE, st));
+        // attention writes its output already rounded to FP8 and packed (the operand of W_o)
+        DS_CHECK(paged_attn_launch(qp, L.k_cache, L.v_cache, block_tables, ctx_after, nullptr, xq, nullptr, pa_scratch, batch, nq,
+                                   nkv, d, dec->block_size, dec->max_blocks, max_ctx, MODE, scale, s));
+        DS_CHECK(gemv(L.w_o, delta, H, nq * d));
         hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, delta, L.norm_mlp,
                            xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
-        DS_CHECK(feather_gemv_fp8_batched(L.w_gate_up, xq, gu, 2 * I, H, batch, MODE, st));
+        DS_CHECK(gemv(L.w_gate_up, gu, 2 * I, H));
         int64_t items = (int64_t)batch * I / 4;
         hipLaunchKernelGGL((swiglu_pack_kernel<MODE>), dim3((unsigned)((items + kDsThreads - 1) / kDsThreads)),
                            dim3(kDsThreads), 0, s, gu, xq, I, batch);
         DS_CHECK(check_launch("feather_decode_step (swiglu)"));
-        DS_CHECK(feather_gemv_fp8_batched(L.w_down, xq, delta, H, I, batch, MODE, st));
+        DS_CHECK(gemv(L.w_down, delta, H, I));
         pending = delta;
     }
     hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending, dec->norm_final,
                        xq, H, dec->rms_eps);
     DS_CHECK(check_launch("feather_decode_step (final norm)"));
-    DS_CHECK(feather_gemv_fp8_batched(dec->w_lm_head, xq, logits, dec->vocab, H, batch, MODE, st));
+    DS_CHECK(gemv(dec->w_lm_head, logits, dec->vocab, H));
 #undef DS_CHECK
     return FEATHER_OK;
 }
@@ -232,7 +211,6 @@ static int64_t step_scratch_bytes(const feather_decoder_t *dec, int64_t batch, i
     t += up(batch * (H > I ? H : I));
     t += up(batch * (nq + 2 * nkv) * d * 4);
     t += up(batch * nq * d);
-    t += up(batch * nq * d * 4);
     t += up(batch * 2 * I * 4);
     t += up(batch * 4);
     t += up(feather_paged_attn_scratch_bytes(batch, nq, d, max_ctx));

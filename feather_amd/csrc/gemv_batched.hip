@@ -8,7 +8,9 @@
 // row across the 4 lanes that share it) and decodes them in registers; the
 // vectors (a few hundred KB at most, L2 resident) are read the same way.
 // One workgroup owns 16 rows; its 4 waves split K and reduce through LDS in a
-// fixed order, so results are deterministic.
+// fixed order, so results are deterministic.  (Handing the vectors over as
+// already-decoded fp16 instead of packed codes was measured and dropped: it
+// doubles the vector bytes every workgroup pulls from L2 and ran 10-40 % slower.)
 #include "common.h"
 
 namespace feather {
@@ -26,7 +28,8 @@ __device__ __forceinline__ half8_t bg_dec8(uint32_t w0, uint32_t w1) {
     return __builtin_bit_cast(half8_t, r);
 }
 
-// K % 256 == 0, w and x 16-byte aligned.  NB = number of 16-vector column blocks.
+// K % 256 == 0 (64 columns per wave step, 4 waves), w and x 16-byte aligned.  NB = number of
+// 16-vector column blocks.
 template <int MODE, int NB>
 __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t *__restrict__ w,
                                                                  const uint8_t *__restrict__ x,
@@ -50,27 +53,25 @@ __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t 
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[nb] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int c = 0; c < kq; c += 128) {        // two 64-column steps in flight
-        u32x4 a0 = load_nt128(wp + c);
-        u32x4 a1 = load_nt128(wp + c + 64);
-        u32x4 b0[NB], b1[NB];
+    constexpr int UN = 4;                      // 64-column steps whose loads are issued together
+    for (int c = 0; c < kq; c += 64 * UN) {
+        u32x4 a[UN], b[UN][NB];
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            b0[nb] = u32x4{0, 0, 0, 0};
-            b1[nb] = u32x4{0, 0, 0, 0};
-            if (xok[nb]) {
-                b0[nb] = *reinterpret_cast<const u32x4 *>(xp[nb] + c);
-                b1[nb] = *reinterpret_cast<const u32x4 *>(xp[nb] + c + 64);
-            }
+        for (int u = 0; u < UN; u++) {
+            const bool in = c + 64 * u < kq;
+            a[u] = in ? load_nt128(wp + c + 64 * u) : u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+                b[u][nb] = in && xok[nb] ? *reinterpret_cast<const u32x4 *>(xp[nb] + c + 64 * u) : u32x4{0, 0, 0, 0};
         }
-        half8_t a00 = bg_dec8<MODE>(a0.x, a0.y), a01 = bg_dec8<MODE>(a0.z, a0.w);
-        half8_t a10 = bg_dec8<MODE>(a1.x, a1.y), a11 = bg_dec8<MODE>(a1.z, a1.w);
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a00, bg_dec8<MODE>(b0[nb].x, b0[nb].y), acc[nb], 0, 0, 0);
-            acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a01, bg_dec8<MODE>(b0[nb].z, b0[nb].w), acc[nb], 0, 0, 0);
-            acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a10, bg_dec8<MODE>(b1[nb].x, b1[nb].y), acc[nb], 0, 0, 0);
-            acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a11, bg_dec8<MODE>(b1[nb].z, b1[nb].w), acc[nb], 0, 0, 0);
+        for (int u = 0; u < UN; u++) {
+            half8_t a0 = bg_dec8<MODE>(a[u].x, a[u].y), a1 = bg_dec8<MODE>(a[u].z, a[u].w);
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bg_dec8<MODE>(b[u][nb].x, b[u][nb].y), acc[nb], 0, 0, 0);
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bg_dec8<MODE>(b[u][nb].z, b[u][nb].w), acc[nb], 0, 0, 0);
+            }
         }
     }
     if (wave > 0) {
@@ -117,7 +118,7 @@ extern "C" int feather_gemv_fp8_batched(const void *w, const void *x, void *out_
     FEATHER_CHECK(w && x && out_f32, FEATHER_EINVAL, "%s: null pointer", me);
     FEATHER_CHECK(aligned(w, 4) && aligned(x, 4) && aligned(out_f32, 16), FEATHER_EINVAL, "%s: misaligned pointer", me);
     hipStream_t s = (hipStream_t)stream;
-    if (K % 512 != 0 || K == 0 || !aligned(w, 16) || !aligned(x, 16)) {
+    if (K % 256 != 0 || K == 0 || !aligned(w, 16) || !aligned(x, 16)) {
         // shapes the MFMA path does not cover: one streaming GEMV per vector
         for (int64_t b = 0; b < nvec; b++) {
             int rc = feather_gemv_fp8(w, (const uint8_t *)x + b * K, (float *)out_f32 + b * M, M, K, mode, stream);

@@ -2,9 +2,12 @@
 // aware.  The kernel is an HBM gather-stream of the K and V blocks; every cache
 // byte is read once per group of query heads that share its KV head.
 //
-// Work split (flash-decoding): one wave per (sequence, KV head, context split).
-// The query heads of the group (up to 16) are the 16 columns of a 16x16 MFMA
-// tile and the tokens are its rows:
+// Work split (flash-decoding): one workgroup of 4 waves per (sequence, KV head,
+// split of 512 tokens); the waves take the 32-token steps of the split round
+// robin and are merged through LDS, the splits of a sequence by a second small
+// kernel (skipped when the whole context fits one split).  Inside a wave the
+// query heads of the group (up to 16) are the 16 columns of a 16x16 MFMA tile
+// and the tokens are its rows:
 //     S^T[tok, qh]  = K[tok, :] . Q[qh, :]
 //     O^T_c[i, qh] += V^T_c[i, tok] P^T[tok, qh],   dd = 4 i + c, c = 0..3
 // K rows are contiguous 16-byte pieces per lane straight from the cache block
@@ -13,14 +16,18 @@
 // lane loads the SAME packed word of 8 tokens and uses byte c of every word
 // for the c-th MFMA (the four bytes of a word are four different head dims),
 // so the transpose is the byte select that decoding does anyway.
-//
-// Each split writes (m, l, unnormalised O) to scratch; a second tiny kernel
-// merges the splits of a (sequence, head).
+// A wave issues the loads of all its steps (up to four) before it consumes the
+// first, so the dependent chains block id -> row address -> data of the steps
+// overlap instead of adding up.
+#include "attention_internal.h"
 #include "common.h"
 
 namespace feather {
 
-constexpr int kSplit = 256;  // tokens per wave
+constexpr int kPaWaves = 4;
+constexpr int kPaThreads = kPaWaves * kWave;
+constexpr int kSplit = 512;   // tokens per workgroup
+constexpr int kStepTok = 32;  // tokens per wave step
 
 __device__ __forceinline__ float4_t pa_mfma16(half8_t a, half8_t b, float4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -55,33 +62,48 @@ __device__ __forceinline__ void v_pairs(uint32_t wa, uint32_t wb, uint32_t out[4
     }
 }
 
-// scratch per (seq, q head, split): [0] = m (log2 domain), [1] = l, [2 .. 2+D) = O
-template <int D, int MODE>
-__global__ __launch_bounds__(64) void paged_attn_split_kernel(
+// scratch per (seq, q head, split): [0] = m (log2 domain), [1] = l, [2 .. 2+D) = unnormalised O
+// FAST: block_size is a power of two >= 4: token -> block / slot by shift and mask, and an aligned
+// group of 4 tokens never straddles a block (one table lookup per group)
+template <int D, int MODE, bool FAST>
+__global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     const uint32_t *__restrict__ q, const uint32_t *__restrict__ k_cache, const uint32_t *__restrict__ v_cache,
     const int32_t *__restrict__ block_tables, const int32_t *__restrict__ ctx_lens, float *__restrict__ scratch,
-    int n_q_heads, int n_kv_heads, int block_size, int max_blocks, int n_splits, int max_ctx, float scale_log2e) {
+    float *__restrict__ out_f32, uint32_t *__restrict__ out_packed, _Float16 *__restrict__ out_q16, int n_q_heads,
+    int n_kv_heads, int block_size, int bs_shift, int max_blocks, int n_splits, int max_ctx, float scale_log2e) {
     constexpr int DW = D / 4;       // words per token row
     constexpr int RB = D / 64;      // 16-word row blocks of V per token
     constexpr int STEPS = D / 32;   // MFMA k-steps of the score product
+    __shared__ float ml_lds[kPaWaves][2][16];
+    __shared__ float4_t o_lds[kPaWaves - 1][RB * 4][kWave];
+
     const int split = blockIdx.x % n_splits;
     const int kvh = (blockIdx.x / n_splits) % n_kv_heads;
     const int seq = blockIdx.x / (n_splits * n_kv_heads);
     const int group = n_q_heads / n_kv_heads;
     const int ctx = min(ctx_lens[seq], max_ctx);  // never index past the block table
     const int t_begin = split * kSplit;
-    const int lane = threadIdx.x, j = lane & 15, kb = lane >> 4;
-    const int t_end = min(t_begin + kSplit, ctx);
-
-    const int qh = kvh * group + j;  // this lane's query head (valid if j < group)
-    float *my = scratch + ((int64_t)(seq * n_q_heads + qh) * n_splits + split) * (D + 2);
-    if (t_begin >= ctx) {            // empty split: neutral element for the merge
-        if (j < group && kb == 0) { my[0] = -INFINITY; my[1] = 0.f; }
+    if (t_begin >= ctx) {                         // empty split: the merge never reads it
+        if (n_splits == 1) {                      // no merge pass: an empty context gives a zero result
+            for (int i = threadIdx.x; i < group * DW; i += kPaThreads) {
+                int64_t w = ((int64_t)seq * n_q_heads + kvh * group) * DW + i;
+                if (out_f32) *reinterpret_cast<float4_t *>(out_f32 + 4 * w) = float4_t{0.f, 0.f, 0.f, 0.f};
+                if (out_packed) out_packed[w] = 0u;
+                if (out_q16) *reinterpret_cast<u32x2 *>(out_q16 + 4 * w) = u32x2{0u, 0u};
+            }
+        }
         return;
     }
+    const int t_end = min(t_begin + kSplit, ctx);
+    const int n_steps = (t_end - t_begin + kStepTok - 1) / kStepTok;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, kb = lane >> 4;
+    auto blk_of = [&](int tok) { return FAST ? tok >> bs_shift : tok / block_size; };
+    auto slot_of = [&](int tok) { return FAST ? tok & (block_size - 1) : tok % block_size; };
 
-    // Q fragments: lane (qh = j, kb) holds dims 16 kb + 8 s' + {0..7} of 32-dim chunk pairs:
-    // k-slot mapping of step st: dims 64 (st / 2) + 16 kb + 8 (st % 2) + {0..7}
+    const int32_t *bt = block_tables + (int64_t)seq * max_blocks;
+
+    const int qh = kvh * group + j;  // this lane's query head (valid if j < group)
+    // Q fragments: k-slot mapping of step st: dims 64 (st / 2) + 16 kb + 8 (st % 2) + {0..7}
     half8_t qf[STEPS];
 #pragma unroll
     for (int st = 0; st < STEPS; st++) {
@@ -98,38 +120,63 @@ __global__ __launch_bounds__(64) void paged_attn_split_kernel(
 #pragma unroll
         for (int c = 0; c < 4; c++) o[rb][c] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
-    const int32_t *bt = block_tables + (int64_t)seq * max_blocks;
 
-    for (int t0 = t_begin; t0 < t_end; t0 += 32) {
-        // ---- scores of 32 tokens: two 16-token row blocks
-        float4_t s[2];
+    // One step = packed K (16 codes of the lane's token per 64-dim chunk) and V (word j of 8 tokens).
+    // Loading is split in two phases so that the table lookups of ALL steps in flight are issued
+    // (and waited for) before the first data load: memory returns in order, so a lookup issued
+    // behind another step's data loads would have to wait for them.
+    struct Step {
+        int64_t kbase[2], vbase[2][4];
+        u32x4 kw[2][RB];
+        uint32_t vw[RB][2][4];
+    };
+    auto row_base = [&](int blk, int tok) { return ((int64_t)blk * n_kv_heads + kvh) * block_size + slot_of(tok); };
+    auto lookup_step = [&](Step &S, int t0) {
 #pragma unroll
         for (int a = 0; a < 2; a++) {
-            int tok = t0 + 16 * a + j;                    // A-operand row of this lane
-            int tc = min(tok, ctx - 1);                   // clamp: masked below
-            int64_t base = ((int64_t)bt[tc / block_size] * n_kv_heads + kvh) * block_size + tc % block_size;
-            const uint32_t *kr = k_cache + base * DW;
-            s[a] = float4_t{0.f, 0.f, 0.f, 0.f};
+            int tc = min(t0 + 16 * a + j, ctx - 1);       // clamp: rows past the context are masked later
+            S.kbase[a] = row_base(bt[blk_of(tc)], tc);
+            if constexpr (FAST) {
+                int tq = min(t0 + 16 * a + 4 * kb, ctx - 1);
+                int64_t qb = row_base(bt[blk_of(tq)], t0 + 16 * a + 4 * kb);
 #pragma unroll
-            for (int c64 = 0; c64 < RB; c64++) {
-                u32x4 w = *reinterpret_cast<const u32x4 *>(kr + 16 * c64 + 4 * kb);  // 16 codes, 64 B per token
-                s[a] = pa_mfma16(pa_dec8<MODE>(w.x, w.y), qf[2 * c64], s[a]);
-                s[a] = pa_mfma16(pa_dec8<MODE>(w.z, w.w), qf[2 * c64 + 1], s[a]);
+                for (int r = 0; r < 4; r++) S.vbase[a][r] = qb + r;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    int tv = min(t0 + 16 * a + 4 * kb + r, ctx - 1);
+                    S.vbase[a][r] = row_base(bt[blk_of(tv)], tv);
+                }
             }
         }
-        // ---- V words: lane (i = j, kb) takes word i of tokens 16 a + 4 kb + r
-        uint32_t vw[RB][2][4];
+    };
+    auto load_step = [&](Step &S, int t0) {
 #pragma unroll
-        for (int a = 0; a < 2; a++)
+        for (int a = 0; a < 2; a++) {
+            const uint32_t *kr = k_cache + S.kbase[a] * DW;
+#pragma unroll
+            for (int c64 = 0; c64 < RB; c64++) S.kw[a][c64] = *reinterpret_cast<const u32x4 *>(kr + 16 * c64 + 4 * kb);
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 int tok = t0 + 16 * a + 4 * kb + r;
-                int tc = min(tok, ctx - 1);
-                int64_t base = ((int64_t)bt[tc / block_size] * n_kv_heads + kvh) * block_size + tc % block_size;
 #pragma unroll
-                for (int rb = 0; rb < RB; rb++) vw[rb][a][r] = tok < ctx ? v_cache[base * DW + 16 * rb + j] : 0u;
+                for (int rb = 0; rb < RB; rb++)
+                    S.vw[rb][a][r] = tok < ctx ? v_cache[S.vbase[a][r] * DW + 16 * rb + j] : 0u;
             }
-        // ---- online softmax (lane column = query head)
+        }
+    };
+    auto compute_step = [&](const Step &S, int t0) {
+        float4_t s[2];
+#pragma unroll
+        for (int a = 0; a < 2; a++) {
+            s[a] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c64 = 0; c64 < RB; c64++) {
+                s[a] = pa_mfma16(pa_dec8<MODE>(S.kw[a][c64].x, S.kw[a][c64].y), qf[2 * c64], s[a]);
+                s[a] = pa_mfma16(pa_dec8<MODE>(S.kw[a][c64].z, S.kw[a][c64].w), qf[2 * c64 + 1], s[a]);
+            }
+        }
+        // online softmax (lane column = query head), log2 domain
         float mx = -INFINITY;
 #pragma unroll
         for (int a = 0; a < 2; a++)
@@ -156,81 +203,207 @@ __global__ __launch_bounds__(64) void paged_attn_split_kernel(
                 p8[4 * a + r] = (_Float16)e;
             }
         l_run = l_run * alpha + rs;
-        // ---- O^T_c += V^T_c P^T
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
             uint32_t pr[4][4];  // [pair index][c]
-            v_pairs<MODE>(vw[rb][0][0], vw[rb][0][1], pr[0]);
-            v_pairs<MODE>(vw[rb][0][2], vw[rb][0][3], pr[1]);
-            v_pairs<MODE>(vw[rb][1][0], vw[rb][1][1], pr[2]);
-            v_pairs<MODE>(vw[rb][1][2], vw[rb][1][3], pr[3]);
+            v_pairs<MODE>(S.vw[rb][0][0], S.vw[rb][0][1], pr[0]);
+            v_pairs<MODE>(S.vw[rb][0][2], S.vw[rb][0][3], pr[1]);
+            v_pairs<MODE>(S.vw[rb][1][0], S.vw[rb][1][1], pr[2]);
+            v_pairs<MODE>(S.vw[rb][1][2], S.vw[rb][1][3], pr[3]);
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 u32x4 vf = u32x4{pr[0][c], pr[1][c], pr[2][c], pr[3][c]};
                 o[rb][c] = pa_mfma16(__builtin_bit_cast(half8_t, vf), p8, o[rb][c] * alpha);
             }
         }
+    };
+
+    {   // The wave's steps are wave, wave + 4, ...  All loads of NF steps are issued before the first
+        // result is needed: a step is a dependent chain (block id -> row address -> data) of several
+        // microseconds, and a wave has only a handful of steps, so they must overlap each other.
+        constexpr int NF = D == 64 ? 4 : (D == 128 ? 2 : 1);
+        Step S[NF];
+        for (int st = wave; st < n_steps; st += kPaWaves * NF) {
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+                if (st + kPaWaves * f < n_steps) lookup_step(S[f], t_begin + kStepTok * (st + kPaWaves * f));
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+                if (st + kPaWaves * f < n_steps) load_step(S[f], t_begin + kStepTok * (st + kPaWaves * f));
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+                if (st + kPaWaves * f < n_steps) compute_step(S[f], t_begin + kStepTok * (st + kPaWaves * f));
+        }
     }
 
-    // ---- write the split's partial: lane (qh = j, kb) holds O rows i = 4 kb + r -> dd = 64 rb + 4 i + c
+    // ---- merge the four waves through LDS (wave 0 finishes)
     float l = l_run;
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
-    if (j < group) {
-        if (kb == 0) { my[0] = m_run; my[1] = l; }
+    if (kb == 0) {
+        ml_lds[wave][0][j] = m_run;
+        ml_lds[wave][1][j] = l;
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) o_lds[wave - 1][rb * 4 + c][lane] = o[rb][c];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float m_all = m_run;
+#pragma unroll
+    for (int w = 1; w < kPaWaves; w++) m_all = fmaxf(m_all, ml_lds[w][0][j]);
+    float wgt = __builtin_amdgcn_exp2f(m_run - m_all);
+    float l_all = wgt * l;
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) o[rb][c] *= wgt;
+#pragma unroll
+    for (int w = 1; w < kPaWaves; w++) {
+        float mw = ml_lds[w][0][j];
+        float ww = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - m_all);
+        l_all += ww * ml_lds[w][1][j];
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[rb][c] += ww * o_lds[w - 1][rb * 4 + c][lane];
+    }
+    if (j >= group) return;
+    // lane (qh = j, kb) holds O rows i = 4 kb + r of every c: dims dd = 64 rb + 4 i + c
+    if (n_splits == 1) {   // the whole context was here: normalise and write the result
+        const float inv = 1.0f / l_all;
+        const int64_t item = (int64_t)seq * n_q_heads + qh;
 #pragma unroll
         for (int rb = 0; rb < RB; rb++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                float4_t x = float4_t{o[rb][0][r], o[rb][1][r], o[rb][2][r], o[rb][3][r]};
-                *reinterpret_cast<float4_t *>(my + 2 + 64 * rb + 4 * (4 * kb + r)) = x;
+                float4_t x = float4_t{o[rb][0][r], o[rb][1][r], o[rb][2][r], o[rb][3][r]} * inv;
+                int w4 = 16 * rb + 4 * kb + r;       // float4 / packed-word index inside the head
+                if (out_f32) *reinterpret_cast<float4_t *>(out_f32 + item * D + 4 * w4) = x;
+                if (out_packed || out_q16) {
+                    const uint32_t word = quant4<MODE>(x[0], x[1], x[2], x[3]);
+                    if (out_packed) out_packed[item * DW + w4] = word;
+                    if (out_q16) *reinterpret_cast<u32x2 *>(out_q16 + item * D + 4 * w4) = dequant4<MODE>(word);
+                }
             }
+        return;
     }
+    float *my = scratch + ((int64_t)(seq * n_q_heads + qh) * n_splits + split) * (D + 2);
+    if (kb == 0) { my[0] = m_all; my[1] = l_all; }
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float4_t x = float4_t{o[rb][0][r], o[rb][1][r], o[rb][2][r], o[rb][3][r]};
+            *reinterpret_cast<float4_t *>(my + 2 + 64 * rb + 4 * (4 * kb + r)) = x;
+        }
 }
 
-// out[seq, qh, :] = sum_s 2^(m_s - m) O_s / sum_s 2^(m_s - m) l_s
-template <int D>
-__global__ __launch_bounds__(64) void paged_attn_merge_kernel(const float *__restrict__ scratch,
-                                                             float *__restrict__ out, int n_splits) {
-    const int64_t item = blockIdx.x;  // seq * n_q_heads + qh
-    const float *base = scratch + item * n_splits * (D + 2);
-    float m = -INFINITY;
-    for (int s = 0; s < n_splits; s++) m = fmaxf(m, base[(int64_t)s * (D + 2)]);
-    float acc[D / 64];
+// out[seq, qh, :] = sum_s 2^(m_s - m) O_s / sum_s 2^(m_s - m) l_s over the splits that hold tokens.
+// One thread per 4 consecutive dims.  Splits are read eight at a time with every load issued
+// before the first use (a loop of dependent loads would pay one memory latency per split).
+template <int D, int MODE>
+__global__ __launch_bounds__(256) void paged_attn_merge_kernel(const float *__restrict__ scratch,
+                                                              const int32_t *__restrict__ ctx_lens,
+                                                              float *__restrict__ out_f32,
+                                                              uint32_t *__restrict__ out_packed,
+                                                              _Float16 *__restrict__ out_q16, int n_items,
+                                                              int n_q_heads, int n_splits, int max_ctx) {
+    constexpr int DW = D / 4;
+    constexpr int G = 8;
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    const int item = gid / DW, w4 = gid % DW;      // item = seq * n_q_heads + qh
+    if (item >= n_items) return;
+    const int ctx = min(ctx_lens[item / n_q_heads], max_ctx);
+    const int used = min(n_splits, (ctx + kSplit - 1) / kSplit);
+    const float *base = scratch + (int64_t)item * n_splits * (D + 2);
+    float m = -INFINITY, l = 0.f;
+    float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < used; s0 += G) {
+        float ms[G], ls[G];
+        float4_t os[G];
 #pragma unroll
-    for (int i = 0; i < D / 64; i++) acc[i] = 0.f;
-    float l = 0.f;
-    for (int s = 0; s < n_splits; s++) {
-        const float *p = base + (int64_t)s * (D + 2);
-        float ms = p[0];
-        if (ms == -INFINITY) continue;
-        float w = __builtin_amdgcn_exp2f(ms - m);
-        l += w * p[1];
+        for (int g = 0; g < G; g++) {
+            const bool in = s0 + g < used;
+            const float *p = base + (int64_t)(in ? s0 + g : 0) * (D + 2);
+            ms[g] = in ? p[0] : -INFINITY;
+            ls[g] = in ? p[1] : 0.f;
+            os[g] = in ? *reinterpret_cast<const float4_t *>(p + 2 + 4 * w4) : float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+        float mg = m;
 #pragma unroll
-        for (int i = 0; i < D / 64; i++) acc[i] += w * p[2 + 64 * i + threadIdx.x];
+        for (int g = 0; g < G; g++) mg = fmaxf(mg, ms[g]);
+        const float keep = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mg);
+        l *= keep;
+        acc *= keep;
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const float w = ms[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms[g] - mg);
+            l += w * ls[g];
+            acc += w * os[g];
+        }
+        m = mg;
     }
-#pragma unroll
-    for (int i = 0; i < D / 64; i++) out[item * D + 64 * i + threadIdx.x] = l > 0.f ? acc[i] / l : 0.f;
+    if (used > 0) acc = acc * (1.0f / l);
+    if (out_f32) *reinterpret_cast<float4_t *>(out_f32 + (int64_t)item * D + 4 * w4) = acc;
+    if (out_packed || out_q16) {
+        const uint32_t word = quant4<MODE>(acc[0], acc[1], acc[2], acc[3]);
+        if (out_packed) out_packed[(int64_t)item * DW + w4] = word;
+        if (out_q16) *reinterpret_cast<u32x2 *>(out_q16 + (int64_t)item * D + 4 * w4) = dequant4<MODE>(word);
+    }
 }
 
 template <int D, int MODE>
-static int launch_paged(const void *q, const void *kc, const void *vc, const void *bt, const void *cl, void *out,
-                        void *scratch, int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads, int64_t block_size,
-                        int64_t max_blocks, int64_t max_ctx, float scale, hipStream_t s) {
+static int launch_paged(const void *q, const void *kc, const void *vc, const void *bt, const void *cl, float *out_f32,
+                        uint32_t *out_packed, _Float16 *out_q16, void *scratch, int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads,
+                        int64_t block_size, int64_t max_blocks, int64_t max_ctx, float scale, hipStream_t s) {
     int n_splits = (int)((max_ctx + kSplit - 1) / kSplit);
     if (n_splits < 1) n_splits = 1;
     int64_t blocks = n_seq * n_kv_heads * n_splits;
     FEATHER_CHECK(blocks < (1ll << 31), FEATHER_ESHAPE, "feather_paged_attn_fp8: grid too large");
+    int bs_shift = -1;
+    for (int sh = 0; sh < 31; sh++)
+        if ((1ll << sh) == block_size) bs_shift = sh;
     const float log2e = 1.4426950408889634f;
-    hipLaunchKernelGGL((paged_attn_split_kernel<D, MODE>), dim3((unsigned)blocks), dim3(64), 0, s,
-                       (const uint32_t *)q, (const uint32_t *)kc, (const uint32_t *)vc, (const int32_t *)bt,
-                       (const int32_t *)cl, (float *)scratch, (int)n_q_heads, (int)n_kv_heads, (int)block_size,
-                       (int)max_blocks, n_splits, (int)max_ctx, scale * log2e);
+    if (bs_shift >= 2)
+        hipLaunchKernelGGL((paged_attn_split_kernel<D, MODE, true>), dim3((unsigned)blocks), dim3(kPaThreads), 0, s,
+                           (const uint32_t *)q, (const uint32_t *)kc, (const uint32_t *)vc, (const int32_t *)bt,
+                           (const int32_t *)cl, (float *)scratch, out_f32, out_packed, out_q16, (int)n_q_heads, (int)n_kv_heads,
+                           (int)block_size, bs_shift, (int)max_blocks, n_splits, (int)max_ctx, scale * log2e);
+    else
+        hipLaunchKernelGGL((paged_attn_split_kernel<D, MODE, false>), dim3((unsigned)blocks), dim3(kPaThreads), 0, s,
+                           (const uint32_t *)q, (const uint32_t *)kc, (const uint32_t *)vc, (const int32_t *)bt,
+                           (const int32_t *)cl, (float *)scratch, out_f32, out_packed, out_q16, (int)n_q_heads, (int)n_kv_heads,
+                           (int)block_size, bs_shift, (int)max_blocks, n_splits, (int)max_ctx, scale * log2e);
     int rc = check_launch("feather_paged_attn_fp8");
-    if (rc != FEATHER_OK) return rc;
-    hipLaunchKernelGGL((paged_attn_merge_kernel<D>), dim3((unsigned)(n_seq * n_q_heads)), dim3(64), 0, s,
-                       (const float *)scratch, (float *)out, n_splits);
+    if (rc != FEATHER_OK || n_splits == 1) return rc;
+    int64_t threads = n_seq * n_q_heads * (D / 4);
+    hipLaunchKernelGGL((paged_attn_merge_kernel<D, MODE>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
+                       (const float *)scratch, (const int32_t *)cl, out_f32, out_packed, out_q16, (int)(n_seq * n_q_heads),
+                       (int)n_q_heads, n_splits, (int)max_ctx);
     return check_launch("feather_paged_attn_fp8 (merge)");
+}
+
+int paged_attn_launch(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,
+                      const void *ctx_lens, float *out_f32, uint32_t *out_packed, _Float16 *out_q16, void *scratch,
+                      int64_t n_seq,
+                      int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
+                      int64_t max_ctx, int mode, float scale, hipStream_t s) {
+#define FEATHER_PA(DD, MM)                                                                                           \
+    return launch_paged<DD, MM>(q, k_cache, v_cache, block_tables, ctx_lens, out_f32, out_packed, out_q16, scratch,  \
+                                n_seq, n_q_heads, n_kv_heads, block_size, max_blocks, max_ctx, scale, s)
+    if (mode == FEATHER_E5M2) {
+        if (d == 64) FEATHER_PA(64, FEATHER_E5M2);
+        if (d == 128) FEATHER_PA(128, FEATHER_E5M2);
+        FEATHER_PA(256, FEATHER_E5M2);
+    }
+    if (d == 64) FEATHER_PA(64, FEATHER_E4M3);
+    if (d == 128) FEATHER_PA(128, FEATHER_E4M3);
+    FEATHER_PA(256, FEATHER_E4M3);
+#undef FEATHER_PA
 }
 
 }  // namespace feather
@@ -264,17 +437,6 @@ extern "C" int feather_paged_attn_fp8(const void *q, const void *k_cache, const 
     FEATHER_CHECK(aligned(q, 8) && aligned(k_cache, 16) && aligned(v_cache, 16) && aligned(out_f32, 4) &&
                       aligned(scratch, 16) && aligned(block_tables, 4) && aligned(ctx_lens, 4),
                   FEATHER_EINVAL, "%s: misaligned pointer", me);
-    hipStream_t s = (hipStream_t)stream;
-#define FEATHER_PA(DD, MM)                                                                                          \
-    return launch_paged<DD, MM>(q, k_cache, v_cache, block_tables, ctx_lens, out_f32, scratch, n_seq, n_q_heads,     \
-                                n_kv_heads, block_size, max_blocks, max_ctx, scale, s)
-    if (mode == FEATHER_E5M2) {
-        if (d == 64) FEATHER_PA(64, FEATHER_E5M2);
-        if (d == 128) FEATHER_PA(128, FEATHER_E5M2);
-        FEATHER_PA(256, FEATHER_E5M2);
-    }
-    if (d == 64) FEATHER_PA(64, FEATHER_E4M3);
-    if (d == 128) FEATHER_PA(128, FEATHER_E4M3);
-    FEATHER_PA(256, FEATHER_E4M3);
-#undef FEATHER_PA
+    return paged_attn_launch(q, k_cache, v_cache, block_tables, ctx_lens, (float *)out_f32, nullptr, nullptr, scratch, n_seq,
+                             n_q_heads, n_kv_heads, d, block_size, max_blocks, max_ctx, mode, scale, (hipStream_t)stream);
 }

@@ -39,35 +39,47 @@ def rope(x: np.ndarray, pos: int, theta: float) -> np.ndarray:
     return np.concatenate([lo * c - hi * s, hi * c + lo * s], axis=-1).astype(np.float32)
 
 
-def online_attention(dots: np.ndarray, V: np.ndarray, scale: float, chunk: int = 32, split: int = 256) -> np.ndarray:
+def online_attention(dots: np.ndarray, V: np.ndarray, scale: float, chunk: int = 32, split: int = 512,
+                     waves: int = 4) -> np.ndarray:
     """Single-query attention with the evaluation order of csrc/paged_attention.hip: tokens in
-    splits of 256, each walked in chunks of 32 with a running maximum (log2 domain), P rounded
-    to fp16 relative to the running maximum for P.V, the denominator summed from the
-    unrounded P, O rescaled when the maximum moves; splits merged at the end.  (Rounding P
-    relative to a running instead of the global maximum moves results by ~2^-12, which is
-    enough to flip an FP8 code downstream, hence the same order here.)"""
+    splits of 512; the 32-token chunks of a split are dealt round robin to 4 waves, each of which
+    keeps a running maximum (log2 domain), rounds P to fp16 relative to it for P.V, sums the
+    denominator from the unrounded P and rescales O when the maximum moves; the waves of a
+    split, then the splits, are merged by their maxima.  (Rounding P relative to a running
+    instead of the global maximum moves results by ~2^-12, which is enough to flip an FP8 code
+    downstream, hence the same order here.)"""
     c = np.float32(scale * 1.4426950408889634)
     x = (dots.astype(np.float32) * c).astype(np.float32)
     n, d = V.shape
-    parts = []
+
+    def merge(parts):
+        parts = [p_ for p_ in parts if np.isfinite(p_[0])]
+        mg = max(p_[0] for p_ in parts)
+        num, den = np.zeros(d, dtype=np.float64), np.float32(0)
+        for m, l, o in parts:
+            w = np.float32(np.exp2(np.float32(m - mg)))
+            num += float(w) * o
+            den = np.float32(den + w * l)
+        return mg, den, num
+
+    split_parts = []
     for s0 in range(0, n, split):
-        m, l, o = -np.inf, np.float32(0), np.zeros(d, dtype=np.float64)
-        for c0 in range(s0, min(s0 + split, n), chunk):
-            xs = x[c0:min(c0 + chunk, n, s0 + split)]
-            m_new = max(m, float(xs.max()))
-            alpha = np.float32(np.exp2(np.float32(m - m_new))) if np.isfinite(m) else np.float32(0)
-            p = np.exp2((xs - np.float32(m_new)).astype(np.float32)).astype(np.float32)
-            l = np.float32(l * alpha + p.sum(dtype=np.float32))
-            o = o * float(alpha) + p.astype(np.float16).astype(np.float64) @ V[c0:c0 + len(xs)]
-            m = m_new
-        parts.append((m, l, o))
-    mg = max(p_[0] for p_ in parts)
-    num, den = np.zeros(d, dtype=np.float64), 0.0
-    for m, l, o in parts:
-        w = float(np.exp2(np.float32(m - mg)))
-        num += w * o
-        den += w * float(l)
-    return (num / den).astype(np.float32)
+        s1 = min(s0 + split, n)
+        wave_parts = []
+        for w in range(waves):
+            m, l, o = -np.inf, np.float32(0), np.zeros(d, dtype=np.float64)
+            for c0 in range(s0 + w * chunk, s1, waves * chunk):
+                xs = x[c0:min(c0 + chunk, s1)]
+                m_new = max(m, float(xs.max()))
+                alpha = np.float32(np.exp2(np.float32(m - m_new))) if np.isfinite(m) else np.float32(0)
+                p = np.exp2((xs - np.float32(m_new)).astype(np.float32)).astype(np.float32)
+                l = np.float32(l * alpha + p.sum(dtype=np.float32))
+                o = o * float(alpha) + p.astype(np.float16).astype(np.float64) @ V[c0:c0 + len(xs)]
+                m = m_new
+            wave_parts.append((m, l, o))
+        split_parts.append(merge(wave_parts))
+    _, den, num = merge(split_parts)
+    return (num / float(den)).astype(np.float32)
 
 
 def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables, ctx_lens, mode: str):

@@ -36,7 +36,7 @@ def test_version_and_error_string():
     assert L.feather_version() >= 100
     assert isinstance(L.feather_last_error(), bytes)
     assert L.feather_dot_scratch_bytes() >= 64 + 4
-    assert L.feather_paged_attn_scratch_bytes(32, 32, 64, 4096) == 32 * 32 * 16 * 66 * 4
+    assert L.feather_paged_attn_scratch_bytes(32, 32, 64, 4096) == 32 * 32 * 8 * 66 * 4
 
 
 def test_c_abi_argument_checks_without_gpu():

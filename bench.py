@@ -177,6 +177,42 @@ def main() -> int:
             extra[f"sdpa_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
             del qkv16, pk
         torch.cuda.empty_cache()
+        # paged-attention decode, 32 sequences x 32 query heads over 4 KV heads, d=64, E4M3, blocks of 16
+        # tokens scattered by a random block table; bytes = K and V codes of every context token once
+        from feather_amd.routines.paged_attention import paged_attention_fp8_acc_fp32_gpu
+        n_seq, Hq, Hkv, d, bs, cmax = 32, 32, 4, 64, 16, 4096
+        nblk = n_seq * cmax // bs
+        kc, vc = (feather.pack_fp8_tensor(randn(nblk * Hkv * bs * d).half(), mode="E4M3").view(nblk, Hkv, bs, d // 4)
+                  for _ in range(2))
+        qp = feather.pack_fp8_tensor(randn(n_seq * Hq * d).half(), mode="E4M3").view(n_seq, Hq, d // 4)
+        bt = torch.randperm(nblk, generator=g, device=dev).to(torch.int32).view(n_seq, cmax // bs)
+        for c in (512, 4096):
+            cl = torch.full((n_seq,), c, dtype=torch.int32, device=dev)
+            us = gpu_time_us(lambda i: paged_attention_fp8_acc_fp32_gpu(qp, kc, vc, bt, cl, mode="E4M3",
+                                                                        max_context_len=c), 50, 5, sync)
+            extra[f"paged_attn_e4m3_s32_h32kv4_d64_ctx{c}_us"] = round(us, 2)
+            extra[f"paged_attn_e4m3_s32_h32kv4_d64_ctx{c}_GBps"] = round(2 * n_seq * Hkv * d * c / us / 1e3, 1)
+        del kc, vc, qp
+        torch.cuda.empty_cache()
+        # decode step of a TinyLlama-1.1B-shaped model (random weights), batch 32, contexts 512..4095, E4M3
+        from feather_amd.routines.decode import TINYLLAMA_1_1B as cfg, PackedDecoder, random_weights
+        wts = random_weights(cfg, seed=5, device=dev)
+        dec = PackedDecoder(cfg, wts, n_blocks=nblk, max_blocks=cmax // bs, mode="E4M3", device=dev)
+        del wts
+        for lay in dec.layers:
+            for name in ("k_cache", "v_cache"):
+                vals = randn(nblk * cfg.n_kv_heads * bs * cfg.head_dim).half()
+                lay[name].view(-1).copy_(feather.pack_fp8_tensor(vals, mode="E4M3").view(torch.int32))
+        cl = torch.randint(512, cmax, (n_seq,), generator=g, device=dev, dtype=torch.int32)
+        tok = torch.randint(0, cfg.vocab, (n_seq,), generator=g, device=dev, dtype=torch.int32)
+        logits = torch.empty((n_seq, cfg.vocab), dtype=torch.float32, device=dev)
+        us = gpu_time_us(lambda i: dec.step(tok, bt, cl, out=logits), 20, 3, sync)
+        step_bytes = dec.weight_bytes() + int(cl.sum().item()) * 2 * cfg.n_kv_heads * cfg.head_dim * cfg.n_layers
+        extra["decode_tinyllama_b32_e4m3_ms_per_step"] = round(us / 1e3, 3)
+        extra["decode_tinyllama_b32_e4m3_tokens_per_s"] = round(n_seq / us * 1e6, 0)
+        extra["decode_tinyllama_b32_e4m3_GBps"] = round(step_bytes / us / 1e3, 1)
+        del dec, logits
+        torch.cuda.empty_cache()
 
     cpu = None
     if not args.no_cpu:

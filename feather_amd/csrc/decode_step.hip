@@ -14,7 +14,7 @@
 // rounded fp32 -> fp16 -> FP8 (RNE, as pack_fp8_tensor does) and packed four
 // codes per word in the producing kernel, so no separate quantisation pass
 // touches memory.  All launches go to one stream; nothing allocates or syncs.
-#include "attention_internal.h"
+#include "internal.h"
 #include "common.h"
 
 namespace feather {
@@ -42,30 +42,75 @@ __global__ __launch_bounds__(kDsThreads) void embed_kernel(const _Float16 *__res
     for (int i = threadIdx.x; i < hidden; i += kDsThreads) h[(int64_t)b * hidden + i] = (float)row[i];
 }
 
+// A GEMV result may arrive as n_part partial sums (slices of K), part_stride floats apart; they
+// are added in slice order.
+__device__ __forceinline__ float4 load_parts(const float *p, int n_part, int64_t part_stride) {
+    constexpr int G = 8;                       // loads in flight: clamped address, unused ones dropped below
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s = 0; s < n_part; s += G) {
+        float4 b[G];
+#pragma unroll
+        for (int u = 0; u < G; u++)
+            b[u] = *reinterpret_cast<const float4 *>(p + (int64_t)min(s + u, n_part - 1) * part_stride);
+        if (s == 0) a = b[0];
+#pragma unroll
+        for (int u = 0; u < G; u++) {
+            if (s + u > 0 && s + u < n_part) { a.x += b[u].x; a.y += b[u].y; a.z += b[u].z; a.w += b[u].w; }
+        }
+    }
+    return a;
+}
+
 // h += delta (if given); xq = pack(fp16(h * rsqrt(mean(h^2) + eps) * w)).  One workgroup per row.
 template <int MODE>
 __global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__restrict__ h,
-                                                                     const float *__restrict__ delta,
+                                                                     const float *__restrict__ delta, int n_part,
+                                                                     int64_t part_stride,
                                                                      const float *__restrict__ w,
                                                                      uint32_t *__restrict__ xq, int hidden,
                                                                      float eps) {
     __shared__ float red[kDsThreads / kWave];
     const int b = blockIdx.x;
     float4 *hr = reinterpret_cast<float4 *>(h + (int64_t)b * hidden);
-    const float4 *dr = delta ? reinterpret_cast<const float4 *>(delta + (int64_t)b * hidden) : nullptr;
+    const float *dr = delta ? delta + (int64_t)b * hidden : nullptr;
     const float4 *wr = reinterpret_cast<const float4 *>(w);
+    // the first kKeep values of a thread stay in registers between the two passes
+    constexpr int kKeep = 4;
+    float4 keep[kKeep];
     float ss = 0.f;
-    for (int i = threadIdx.x; i < hidden / 4; i += kDsThreads) {
+#pragma unroll
+    for (int it = 0; it < kKeep; it++) {
+        const int i = threadIdx.x + it * kDsThreads;
+        if (i < hidden / 4) {
+            float4 x = hr[i];
+            if (dr) {
+                float4 d = load_parts(dr + 4 * i, n_part, part_stride);
+                x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
+                hr[i] = x;
+            }
+            keep[it] = x;
+            ss += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+        }
+    }
+    for (int i = threadIdx.x + kKeep * kDsThreads; i < hidden / 4; i += kDsThreads) {
         float4 x = hr[i];
         if (dr) {
-            float4 d = dr[i];
+            float4 d = load_parts(dr + 4 * i, n_part, part_stride);
             x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
             hr[i] = x;
         }
         ss += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
     }
     const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
-    for (int i = threadIdx.x; i < hidden / 4; i += kDsThreads) {
+#pragma unroll
+    for (int it = 0; it < kKeep; it++) {
+        const int i = threadIdx.x + it * kDsThreads;
+        if (i < hidden / 4) {
+            float4 x = keep[it], g = wr[i];
+            xq[(int64_t)b * (hidden / 4) + i] = quant4<MODE>(x.x * r * g.x, x.y * r * g.y, x.z * r * g.z, x.w * r * g.w);
+        }
+    }
+    for (int i = threadIdx.x + kKeep * kDsThreads; i < hidden / 4; i += kDsThreads) {
         float4 x = hr[i], g = wr[i];
         xq[(int64_t)b * (hidden / 4) + i] = quant4<MODE>(x.x * r * g.x, x.y * r * g.y, x.z * r * g.z, x.w * r * g.w);
     }
@@ -73,14 +118,15 @@ __global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__r
 
 // gu [B, 2 * inter] (gate rows then up rows) -> pack(fp16(silu(gate) * up)) [B, inter / 4]
 template <int MODE>
-__global__ __launch_bounds__(kDsThreads) void swiglu_pack_kernel(const float *__restrict__ gu,
+__global__ __launch_bounds__(kDsThreads) void swiglu_pack_kernel(const float *__restrict__ gu, int n_part,
+                                                                int64_t part_stride,
                                                                 uint32_t *__restrict__ out, int inter, int batch) {
     const int per_row = inter / 4;
     for (int64_t i = (int64_t)blockIdx.x * kDsThreads + threadIdx.x; i < (int64_t)batch * per_row;
          i += (int64_t)gridDim.x * kDsThreads) {
         int b = (int)(i / per_row), c = (int)(i % per_row);
-        float4 g = reinterpret_cast<const float4 *>(gu + (int64_t)b * 2 * inter)[c];
-        float4 u = reinterpret_cast<const float4 *>(gu + (int64_t)b * 2 * inter + inter)[c];
+        float4 g = load_parts(gu + (int64_t)b * 2 * inter + 4 * c, n_part, part_stride);
+        float4 u = load_parts(gu + (int64_t)b * 2 * inter + inter + 4 * c, n_part, part_stride);
         auto f = [](float a, float bb) { return a / (1.0f + expf(-a)) * bb; };
         out[i] = quant4<MODE>(f(g.x, u.x), f(g.y, u.y), f(g.z, u.z), f(g.w, u.w));
     }
@@ -89,8 +135,10 @@ __global__ __launch_bounds__(kDsThreads) void swiglu_pack_kernel(const float *__
 // qkv [B, (n_q + 2 n_kv) * d] fp32 -> RoPE on q and k (rotate-half convention: element j pairs
 // with j + d/2, angle pos * theta^(-2j/d)), q packed to qp [B, n_q, d/4], k and v encoded and
 // written into the paged cache at position pos = ctx_lens[b]; ctx_after[b] = pos + 1.
+constexpr int kRopeThreads = 64;
 template <int MODE>
-__global__ __launch_bounds__(kDsThreads) void rope_append_kernel(const float *__restrict__ qkv,
+__global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *__restrict__ qkv, int n_part,
+                                                                int64_t part_stride,
                                                                 uint32_t *__restrict__ qp,
                                                                 uint32_t *__restrict__ k_cache,
                                                                 uint32_t *__restrict__ v_cache,
@@ -100,16 +148,20 @@ __global__ __launch_bounds__(kDsThreads) void rope_append_kernel(const float *__
                                                                 int d, int block_size, int max_blocks,
                                                                 float log2_theta) {
     const int b = blockIdx.x;
-    const int pos = min(ctx_lens[b], max_blocks * block_size - 1);
-    if (threadIdx.x == 0) ctx_after[b] = pos + 1;
     const int dw = d / 4, half_w = d / 8;            // words per head, words per rotation half
     const int heads = n_q + 2 * n_kv;
+    const int item = blockIdx.y * kRopeThreads + threadIdx.x;
+    const bool live = item < heads * half_w;
+    const int head = live ? item / half_w : 0, t = live ? item % half_w : 0;
+    // the GEMV partials do not depend on the position: their loads go out before the lookups below
+    const float *x = qkv + ((int64_t)b * heads + head) * d;
+    float4 lo = load_parts(x + 4 * t, n_part, part_stride);          // elements 4t .. 4t+3
+    float4 hi = load_parts(x + d / 2 + 4 * t, n_part, part_stride);  // their partners
+    const int pos = min(ctx_lens[b], max_blocks * block_size - 1);
+    if (threadIdx.x == 0 && blockIdx.y == 0) ctx_after[b] = pos + 1;
     const int64_t slot = ((int64_t)block_tables[(int64_t)b * max_blocks + pos / block_size] * n_kv) * block_size;
-    for (int item = threadIdx.x; item < heads * half_w; item += kDsThreads) {
-        const int head = item / half_w, t = item % half_w;
-        const float *x = qkv + ((int64_t)b * heads + head) * d;
-        float4 lo = reinterpret_cast<const float4 *>(x)[t];              // elements 4t .. 4t+3
-        float4 hi = reinterpret_cast<const float4 *>(x + d / 2)[t];      // their partners
+    if (!live) return;
+    {
         if (head < n_q + n_kv) {
             float lo4[4] = {lo.x, lo.y, lo.z, lo.w}, hi4[4] = {hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
@@ -138,28 +190,75 @@ __global__ __launch_bounds__(kDsThreads) void rope_append_kernel(const float *__
     }
 }
 
+// K slices per GEMV: enough 64-row tiles x slices to cover the 256 CUs, at most one slice per
+// 256-column chunk (the launcher's own clamp, repeated here to size the partial buffers)
+static int plan_splits(int64_t M, int64_t K) {
+    if (K % 256 != 0 || K == 0) return 1;          // the per-vector fallback writes complete sums
+    const int64_t tiles = (M + 63) / 64, n_chunks = K / 256;
+    static const int target = getenv("FEATHER_BG_TARGET") ? atoi(getenv("FEATHER_BG_TARGET")) : 256;
+    int64_t s = (target + tiles - 1) / tiles;
+    s = s < 1 ? 1 : (s > 16 ? 16 : s);
+    s = s > n_chunks ? n_chunks : s;
+    const int64_t cps = (n_chunks + s - 1) / s;
+    return (int)((n_chunks + cps - 1) / cps);
+}
+
+struct StepPlan {
+    int s_qkv, s_o, s_gu, s_down;
+    int64_t qkv_rows;
+    size_t b_h, b_delta, b_xq, b_qkv, b_qp, b_gu, b_ctx;
+};
+
+static StepPlan plan_step(const feather_decoder_t *dec, int64_t batch) {
+    const int64_t H = dec->hidden, nq = dec->n_q_heads, nkv = dec->n_kv_heads, d = dec->head_dim, I = dec->inter;
+    StepPlan P;
+    P.qkv_rows = (nq + 2 * nkv) * d;
+    P.s_qkv = plan_splits(P.qkv_rows, H);
+    P.s_o = plan_splits(H, nq * d);
+    P.s_gu = plan_splits(2 * I, H);
+    P.s_down = plan_splits(H, I);
+    auto up = [](int64_t b) { return (size_t)((b + 255) / 256 * 256); };
+    P.b_h = up(batch * H * 4);
+    P.b_delta = up((int64_t)(P.s_o > P.s_down ? P.s_o : P.s_down) * batch * H * 4);
+    P.b_xq = up(batch * (H > I ? H : I));
+    P.b_qkv = up((int64_t)P.s_qkv * batch * P.qkv_rows * 4);
+    P.b_qp = up(batch * nq * d);
+    P.b_gu = up((int64_t)P.s_gu * batch * 2 * I * 4);
+    P.b_ctx = up(batch * 4);
+    return P;
+}
+
 template <int MODE>
 static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const int32_t *block_tables,
                     const int32_t *ctx_lens, int batch, int max_ctx, void *scratch, float *logits, hipStream_t s) {
     const int H = dec->hidden, nq = dec->n_q_heads, nkv = dec->n_kv_heads, d = dec->head_dim, I = dec->inter;
-    const int qkv_rows = (nq + 2 * nkv) * d;
+    const StepPlan P = plan_step(dec, batch);
+    const int qkv_rows = (int)P.qkv_rows;
     // scratch carve-up (all offsets multiples of 256 bytes)
     char *p = (char *)scratch;
-    auto take = [&](size_t bytes) { char *q = p; p += (bytes + 255) / 256 * 256; return q; };
-    float *h = (float *)take((size_t)batch * H * 4);
-    float *delta = (float *)take((size_t)batch * H * 4);
-    uint32_t *xq = (uint32_t *)take((size_t)batch * (H > I ? H : I));
-    float *qkv = (float *)take((size_t)batch * qkv_rows * 4);
-    uint32_t *qp = (uint32_t *)take((size_t)batch * nq * d);
-    float *gu = (float *)take((size_t)batch * 2 * I * 4);
-    int32_t *ctx_after = (int32_t *)take((size_t)batch * 4);
+    auto take = [&](size_t bytes) { char *q = p; p += bytes; return q; };
+    float *h = (float *)take(P.b_h);
+    float *delta = (float *)take(P.b_delta);
+    uint32_t *xq = (uint32_t *)take(P.b_xq);
+    float *qkv = (float *)take(P.b_qkv);
+    uint32_t *qp = (uint32_t *)take(P.b_qp);
+    float *gu = (float *)take(P.b_gu);
+    int32_t *ctx_after = (int32_t *)take(P.b_ctx);
     void *pa_scratch = p;
     const float scale = 1.0f / sqrtf((float)d);
     const float log2_theta = log2f(dec->rope_theta);
     void *st = (void *)s;
     int rc;
-    auto gemv = [&](const void *w, float *out, int M, int K) {
-        return feather_gemv_fp8_batched(w, xq, out, M, K, batch, MODE, st);
+    // out receives `splits` partial results of [batch, M], batch * M floats apart
+    auto gemv = [&](const void *w, float *out, int M, int K, int splits) {
+        if (K % 256 != 0) return feather_gemv_fp8_batched(w, xq, out, M, K, batch, MODE, st);
+        int got = 0;
+        int r = gemv_batched_launch(w, xq, out, M, K, batch, MODE, splits, (int64_t)batch * M, &got, s);
+        if (r == FEATHER_OK && got != splits) {
+            set_error("feather_decode_step: GEMV slice plan mismatch (%d vs %d)", got, splits);
+            return (int)FEATHER_EINVAL;
+        }
+        return r;
     };
 #define DS_CHECK(call)            \
     do {                          \
@@ -170,51 +269,46 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
     hipLaunchKernelGGL(embed_kernel, dim3(batch), dim3(kDsThreads), 0, s, (const _Float16 *)dec->embed_f16, tokens, h, H);
     DS_CHECK(check_launch("feather_decode_step (embed)"));
     const float *pending = nullptr;                       // output of the previous down projection, not yet added
+    const int64_t hs = (int64_t)batch * H;
     for (int l = 0; l < dec->n_layers; l++) {
         const feather_decoder_layer_t &L = dec->layers[l];
-        hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending,
+        hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending, P.s_down, hs,
                            L.norm_attn, xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
-        DS_CHECK(gemv(L.w_qkv, qkv, qkv_rows, H));
-        hipLaunchKernelGGL((rope_append_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, qkv, qp,
-                           (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, block_tables, ctx_lens, ctx_after, nq, nkv, d,
-                           dec->block_size, dec->max_blocks, log2_theta);
+        DS_CHECK(gemv(L.w_qkv, qkv, qkv_rows, H, P.s_qkv));
+        hipLaunchKernelGGL((rope_append_kernel<MODE>),
+                           dim3(batch, ((nq + 2 * nkv) * (d / 8) + kRopeThreads - 1) / kRopeThreads), dim3(kRopeThreads), 0, s, qkv, P.s_qkv,
+                           (int64_t)batch * qkv_rows, qp, (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, block_tables,
+                           ctx_lens, ctx_after, nq, nkv, d, dec->block_size, dec->max_blocks, log2_theta);
         DS_CHECK(check_launch("feather_decode_step (rope)"));
         // attention writes its output already rounded to FP8 and packed (the operand of W_o)
         DS_CHECK(paged_attn_launch(qp, L.k_cache, L.v_cache, block_tables, ctx_after, nullptr, xq, nullptr, pa_scratch, batch, nq,
                                    nkv, d, dec->block_size, dec->max_blocks, max_ctx, MODE, scale, s));
-        DS_CHECK(gemv(L.w_o, delta, H, nq * d));
-        hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, delta, L.norm_mlp,
-                           xq, H, dec->rms_eps);
+        DS_CHECK(gemv(L.w_o, delta, H, nq * d, P.s_o));
+        hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, delta, P.s_o, hs,
+                           L.norm_mlp, xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
-        DS_CHECK(gemv(L.w_gate_up, gu, 2 * I, H));
+        DS_CHECK(gemv(L.w_gate_up, gu, 2 * I, H, P.s_gu));
         int64_t items = (int64_t)batch * I / 4;
         hipLaunchKernelGGL((swiglu_pack_kernel<MODE>), dim3((unsigned)((items + kDsThreads - 1) / kDsThreads)),
-                           dim3(kDsThreads), 0, s, gu, xq, I, batch);
+                           dim3(kDsThreads), 0, s, gu, P.s_gu, (int64_t)batch * 2 * I, xq, I, batch);
         DS_CHECK(check_launch("feather_decode_step (swiglu)"));
-        DS_CHECK(gemv(L.w_down, delta, H, I));
+        DS_CHECK(gemv(L.w_down, delta, H, I, P.s_down));
         pending = delta;
     }
-    hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending, dec->norm_final,
-                       xq, H, dec->rms_eps);
+    hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending, P.s_down, hs,
+                       dec->norm_final, xq, H, dec->rms_eps);
     DS_CHECK(check_launch("feather_decode_step (final norm)"));
-    DS_CHECK(gemv(dec->w_lm_head, logits, dec->vocab, H));
+    DS_CHECK(feather_gemv_fp8_batched(dec->w_lm_head, xq, logits, dec->vocab, H, batch, MODE, st));
 #undef DS_CHECK
     return FEATHER_OK;
 }
 
 static int64_t step_scratch_bytes(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx) {
-    const int64_t H = dec->hidden, nq = dec->n_q_heads, nkv = dec->n_kv_heads, d = dec->head_dim, I = dec->inter;
+    const StepPlan P = plan_step(dec, batch);
     auto up = [](int64_t b) { return (b + 255) / 256 * 256; };
-    int64_t t = 0;
-    t += 2 * up(batch * H * 4);
-    t += up(batch * (H > I ? H : I));
-    t += up(batch * (nq + 2 * nkv) * d * 4);
-    t += up(batch * nq * d);
-    t += up(batch * 2 * I * 4);
-    t += up(batch * 4);
-    t += up(feather_paged_attn_scratch_bytes(batch, nq, d, max_ctx));
-    return t;
+    return (int64_t)(P.b_h + P.b_delta + P.b_xq + P.b_qkv + P.b_qp + P.b_gu + P.b_ctx) +
+           up(feather_paged_attn_scratch_bytes(batch, dec->n_q_heads, dec->head_dim, max_ctx));
 }
 
 }  // namespace feather

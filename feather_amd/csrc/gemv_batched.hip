@@ -3,19 +3,30 @@
 //
 // With more than a couple of vectors the per-element multiply count rules out
 // the VALU, so the product runs on the matrix cores: a 16-row slab of W is the
-// A operand of v_mfma_f32_16x16x32_f16 and 16 vectors are the B columns.  A
-// lane loads 16 consecutive codes of one row (128-bit load, 64 B contiguous per
-// row across the 4 lanes that share it) and decodes them in registers; the
-// vectors (a few hundred KB at most, L2 resident) are read the same way.
-// One workgroup owns 16 rows; its 4 waves split K and reduce through LDS in a
-// fixed order, so results are deterministic.  (Handing the vectors over as
-// already-decoded fp16 instead of packed codes was measured and dropped: it
-// doubles the vector bytes every workgroup pulls from L2 and ran 10-40 % slower.)
+// A operand of v_mfma_f32_16x16x32_f16 and 16 vectors are the B columns.
+// A workgroup of 4 waves owns 64 rows (16 per wave) and a slice of K, walked in
+// chunks of 256 columns.  Per chunk every lane loads 4 x 16 consecutive codes
+// of its row (128-bit loads) and decodes them in registers; the vectors' chunk
+// is decoded ONCE per workgroup into LDS as fp16 (each thread 16 codes per 16
+// vectors) and read from there as the B operand by all four waves, so the
+// vector bytes pulled from L2 and their decode cost a quarter of the weight's
+// instead of twice as much with one 16-row slab per workgroup.  The loads of
+// chunk c + 1 are issued before the MFMAs of chunk c; LDS is double buffered,
+// one barrier per chunk.
+// Small matrices do not have enough 64-row tiles to fill 256 CUs; the internal
+// launcher therefore cuts K into slices that write separate partial results
+// which the consumer adds in slice order (deterministic, no atomics).
+// (Handing the vectors over as already-decoded fp16 instead of packed codes was
+// measured and dropped: it doubles the vector bytes pulled from L2.)
 #include "common.h"
+#include "internal.h"
 
 namespace feather {
 
 constexpr int kBgThreads = 256;
+constexpr int kBgChunk = 256;                  // columns per chunk
+constexpr int kBgPitch = kBgChunk + 8;         // halfs per LDS row: +16 B keeps 8 lanes x 16 B on distinct banks
+constexpr int kBgRows = 64;                    // rows per workgroup
 
 template <int MODE>
 __device__ __forceinline__ half8_t bg_dec8(uint32_t w0, uint32_t w1) {
@@ -28,78 +39,125 @@ __device__ __forceinline__ half8_t bg_dec8(uint32_t w0, uint32_t w1) {
     return __builtin_bit_cast(half8_t, r);
 }
 
-// K % 256 == 0 (64 columns per wave step, 4 waves), w and x 16-byte aligned.  NB = number of
-// 16-vector column blocks.
+// K % 256 == 0, w and x 16-byte aligned.  NB = number of 16-vector column blocks.
+// grid = (row tiles, K slices); slice s covers chunks [s * cps, min((s + 1) * cps, K / 256)).
 template <int MODE, int NB>
 __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t *__restrict__ w,
                                                                  const uint8_t *__restrict__ x,
-                                                                 float *__restrict__ out, int M, int K, int nvec) {
-    __shared__ float4_t red[3][NB][kWave];
+                                                                 float *__restrict__ out, int M, int K, int nvec,
+                                                                 int cps, int64_t part_stride) {
+    extern __shared__ __attribute__((aligned(16))) _Float16 xs[];   // [2][16 * NB][kBgPitch]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 15, kb = lane >> 4;
-    const int row0 = blockIdx.x * 16;
+    const int row0 = blockIdx.x * kBgRows + 16 * wave;
     const int row = min(row0 + j, M - 1);
-    const int kq = K / 4;                      // this wave's share of K
-    const uint8_t *wp = w + (int64_t)row * K + wave * kq + 16 * kb;
+    const int n_chunks = K / kBgChunk;
+    const int c_begin = blockIdx.y * cps, c_end = min(c_begin + cps, n_chunks);
+    const uint8_t *wp = w + (int64_t)row * K + 16 * kb;
+    // this thread's share of the vectors' chunk: 16-byte piece (vec, col16) = (piece / 16, piece % 16)
     const uint8_t *xp[NB];
     bool xok[NB];
+    int xdst[NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) {
-        int vec = 16 * nb + j;
-        xok[nb] = vec < nvec;
-        xp[nb] = x + (int64_t)min(vec, nvec - 1) * K + wave * kq + 16 * kb;
+    for (int i = 0; i < NB; i++) {
+        int piece = threadIdx.x + kBgThreads * i;
+        int vec = piece >> 4, col16 = piece & 15;
+        xok[i] = vec < nvec;
+        xp[i] = x + (int64_t)min(vec, nvec - 1) * K + 16 * col16;
+        xdst[i] = vec * kBgPitch + 16 * col16;
     }
     float4_t acc[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[nb] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    constexpr int UN = 4;                      // 64-column steps whose loads are issued together
-    for (int c = 0; c < kq; c += 64 * UN) {
-        u32x4 a[UN], b[UN][NB];
+    u32x4 wa[4], xa[NB];
+    auto issue = [&](int c, u32x4 (&wr)[4], u32x4 (&xr)[NB]) {
+        const int64_t col = (int64_t)c * kBgChunk;
 #pragma unroll
-        for (int u = 0; u < UN; u++) {
-            const bool in = c + 64 * u < kq;
-            a[u] = in ? load_nt128(wp + c + 64 * u) : u32x4{0, 0, 0, 0};
+        for (int u = 0; u < 4; u++) wr[u] = load_nt128(wp + col + 64 * u);
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++)
-                b[u][nb] = in && xok[nb] ? *reinterpret_cast<const u32x4 *>(xp[nb] + c + 64 * u) : u32x4{0, 0, 0, 0};
+        for (int i = 0; i < NB; i++) xr[i] = xok[i] ? *reinterpret_cast<const u32x4 *>(xp[i] + col) : u32x4{0, 0, 0, 0};
+    };
+    if (c_begin < c_end) issue(c_begin, wa, xa);
+    for (int c = c_begin; c < c_end; c++) {
+        _Float16 *buf = xs + ((c - c_begin) & 1) * (16 * NB * kBgPitch);
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            *reinterpret_cast<half8_t *>(buf + xdst[i]) = bg_dec8<MODE>(xa[i].x, xa[i].y);
+            *reinterpret_cast<half8_t *>(buf + xdst[i] + 8) = bg_dec8<MODE>(xa[i].z, xa[i].w);
         }
+        u32x4 wn[4], xn[NB];
+        if (c + 1 < c_end) issue(c + 1, wn, xn);
+        __syncthreads();
 #pragma unroll
-        for (int u = 0; u < UN; u++) {
-            half8_t a0 = bg_dec8<MODE>(a[u].x, a[u].y), a1 = bg_dec8<MODE>(a[u].z, a[u].w);
+        for (int u = 0; u < 4; u++) {
+            half8_t a0 = bg_dec8<MODE>(wa[u].x, wa[u].y), a1 = bg_dec8<MODE>(wa[u].z, wa[u].w);
 #pragma unroll
             for (int nb = 0; nb < NB; nb++) {
-                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bg_dec8<MODE>(b[u][nb].x, b[u][nb].y), acc[nb], 0, 0, 0);
-                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bg_dec8<MODE>(b[u][nb].z, b[u][nb].w), acc[nb], 0, 0, 0);
+                const _Float16 *b = buf + (16 * nb + j) * kBgPitch + 64 * u + 16 * kb;
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, *reinterpret_cast<const half8_t *>(b), acc[nb], 0, 0, 0);
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, *reinterpret_cast<const half8_t *>(b + 8), acc[nb], 0, 0, 0);
+            }
+        }
+        if (c + 1 < c_end) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) wa[u] = wn[u];
+#pragma unroll
+            for (int i = 0; i < NB; i++) xa[i] = xn[i];
+        }
+    }
+    float *o_base = out + (int64_t)blockIdx.y * part_stride;
+    const int r = row0 + 4 * kb;                   // accumulator rows 4 kb + {0..3}, column = vector
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        int vec = 16 * nb + j;
+        if (vec < nvec) {
+            float *o = o_base + (int64_t)vec * M + r;
+            if (r + 3 < M && (M & 3) == 0) {
+                *reinterpret_cast<float4_t *>(o) = acc[nb];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (r + i < M) o[i] = acc[nb][i];
             }
         }
     }
-    if (wave > 0) {
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) red[wave - 1][nb][lane] = acc[nb];
-    }
-    __syncthreads();
-    if (wave == 0) {
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            float4_t s = acc[nb];
-            s += red[0][nb][lane];
-            s += red[1][nb][lane];
-            s += red[2][nb][lane];
-            int vec = 16 * nb + j;
-            int r = row0 + 4 * kb;             // accumulator rows 4 kb + {0..3}, column = vector
-            if (vec < nvec) {
-                float *o = out + (int64_t)vec * M + r;
-                if (r + 3 < M && (M & 3) == 0) {
-                    *reinterpret_cast<float4_t *>(o) = s;
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        if (r + i < M) o[i] = s[i];
-                }
-            }
+}
+
+template <int MODE, int NB>
+static void bg_launch(const void *w, const void *x, float *out, int M, int K, int nvec, int splits, int cps,
+                      int64_t part_stride, hipStream_t s) {
+    const size_t lds = (size_t)2 * 16 * NB * kBgPitch * sizeof(_Float16);
+    if (lds > 64 * 1024) {
+        static bool raised = false;                // once per process: allow more than 64 KB of dynamic LDS
+        if (!raised) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_batched_kernel<MODE, NB>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            raised = true;
         }
     }
+    hipLaunchKernelGGL((gemv_batched_kernel<MODE, NB>), dim3((unsigned)((M + kBgRows - 1) / kBgRows), (unsigned)splits),
+                       dim3(kBgThreads), lds, s, (const uint8_t *)w, (const uint8_t *)x, out, M, K, nvec, cps, part_stride);
+}
+
+int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M, int64_t K, int64_t nvec, int mode,
+                        int splits, int64_t part_stride, int *splits_out, hipStream_t stream) {
+    const int n_chunks = (int)(K / kBgChunk);
+    splits = splits < 1 ? 1 : (splits > n_chunks ? n_chunks : splits);
+    const int cps = (n_chunks + splits - 1) / splits;
+    splits = (n_chunks + cps - 1) / cps;           // no empty slice
+    if (splits_out) *splits_out = splits;
+    const int nb = (int)((nvec + 15) / 16);
+#define FEATHER_BG(MM, NBB) bg_launch<MM, NBB>(w, x, out_f32, (int)M, (int)K, (int)nvec, splits, cps, part_stride, stream)
+    if (mode == FEATHER_E5M2) {
+        switch (nb) { case 1: FEATHER_BG(FEATHER_E5M2, 1); break; case 2: FEATHER_BG(FEATHER_E5M2, 2); break;
+                      case 3: FEATHER_BG(FEATHER_E5M2, 3); break; default: FEATHER_BG(FEATHER_E5M2, 4); }
+    } else {
+        switch (nb) { case 1: FEATHER_BG(FEATHER_E4M3, 1); break; case 2: FEATHER_BG(FEATHER_E4M3, 2); break;
+                      case 3: FEATHER_BG(FEATHER_E4M3, 3); break; default: FEATHER_BG(FEATHER_E4M3, 4); }
+    }
+#undef FEATHER_BG
+    return check_launch("feather_gemv_fp8_batched");
 }
 
 }  // namespace feather
@@ -117,8 +175,7 @@ extern "C" int feather_gemv_fp8_batched(const void *w, const void *x, void *out_
     if (M == 0) return FEATHER_OK;
     FEATHER_CHECK(w && x && out_f32, FEATHER_EINVAL, "%s: null pointer", me);
     FEATHER_CHECK(aligned(w, 4) && aligned(x, 4) && aligned(out_f32, 16), FEATHER_EINVAL, "%s: misaligned pointer", me);
-    hipStream_t s = (hipStream_t)stream;
-    if (K % 256 != 0 || K == 0 || !aligned(w, 16) || !aligned(x, 16)) {
+    if (K % kBgChunk != 0 || K == 0 || !aligned(w, 16) || !aligned(x, 16)) {
         // shapes the MFMA path does not cover: one streaming GEMV per vector
         for (int64_t b = 0; b < nvec; b++) {
             int rc = feather_gemv_fp8(w, (const uint8_t *)x + b * K, (float *)out_f32 + b * M, M, K, mode, stream);
@@ -126,18 +183,5 @@ extern "C" int feather_gemv_fp8_batched(const void *w, const void *x, void *out_
         }
         return FEATHER_OK;
     }
-    unsigned blocks = (unsigned)((M + 15) / 16);
-    int nb = (int)((nvec + 15) / 16);
-#define FEATHER_BG(MM, NBB)                                                                                        \
-    hipLaunchKernelGGL((gemv_batched_kernel<MM, NBB>), dim3(blocks), dim3(kBgThreads), 0, s, (const uint8_t *)w,  \
-                       (const uint8_t *)x, (float *)out_f32, (int)M, (int)K, (int)nvec)
-    if (mode == FEATHER_E5M2) {
-        switch (nb) { case 1: FEATHER_BG(FEATHER_E5M2, 1); break; case 2: FEATHER_BG(FEATHER_E5M2, 2); break;
-                      case 3: FEATHER_BG(FEATHER_E5M2, 3); break; default: FEATHER_BG(FEATHER_E5M2, 4); }
-    } else {
-        switch (nb) { case 1: FEATHER_BG(FEATHER_E4M3, 1); break; case 2: FEATHER_BG(FEATHER_E4M3, 2); break;
-                      case 3: FEATHER_BG(FEATHER_E4M3, 3); break; default: FEATHER_BG(FEATHER_E4M3, 4); }
-    }
-#undef FEATHER_BG
-    return check_launch(me);
+    return gemv_batched_launch(w, x, (float *)out_f32, M, K, nvec, mode, 1, 0, nullptr, (hipStream_t)stream);
 }

@@ -15,4 +15,11 @@ int paged_attn_launch(const void *q, const void *k_cache, const void *v_cache, c
                       int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
                       int64_t max_ctx, int mode, float scale, hipStream_t stream);
 
+// Batched GEMV with the K range cut into `splits` slices: slice s writes its partial sums to
+// out_f32 + s * part_stride ([nvec, M] each); the consumer adds the slices in index order.
+// Needs K % 256 == 0 and 16-byte aligned w and x; splits is clamped to K / 256.  Returns the
+// number of slices actually written through *splits_out.
+int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M, int64_t K, int64_t nvec, int mode,
+                        int splits, int64_t part_stride, int *splits_out, hipStream_t stream);
+
 }  // namespace feather

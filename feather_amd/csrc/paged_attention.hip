@@ -19,7 +19,7 @@
 // A wave issues the loads of all its steps (up to four) before it consumes the
 // first, so the dependent chains block id -> row address -> data of the steps
 // overlap instead of adding up.
-#include "attention_internal.h"
+#include "internal.h"
 #include "common.h"
 
 namespace feather {
@@ -81,8 +81,56 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     const int kvh = (blockIdx.x / n_splits) % n_kv_heads;
     const int seq = blockIdx.x / (n_splits * n_kv_heads);
     const int group = n_q_heads / n_kv_heads;
-    const int ctx = min(ctx_lens[seq], max_ctx);  // never index past the block table
+    const int ctx_raw = ctx_lens[seq];
     const int t_begin = split * kSplit;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, kb = lane >> 4;
+    auto blk_of = [&](int tok) { return FAST ? tok >> bs_shift : tok / block_size; };
+    auto slot_of = [&](int tok) { return FAST ? tok & (block_size - 1) : tok % block_size; };
+    const int32_t *bt = block_tables + (int64_t)seq * max_blocks;
+
+    const int qh = kvh * group + j;  // this lane's query head (valid if j < group)
+    // Q fragments: k-slot mapping of step st: dims 64 (st / 2) + 16 kb + 8 (st % 2) + {0..7}
+    u32x2 qw[STEPS];
+#pragma unroll
+    for (int st = 0; st < STEPS; st++) {
+        qw[st] = u32x2{0, 0};
+        if (j < group)
+            qw[st] = *reinterpret_cast<const u32x2 *>(q + (int64_t)(seq * n_q_heads + qh) * DW + 16 * (st / 2) + 4 * kb +
+                                                      2 * (st % 2));
+    }
+
+    // One step = packed K (16 codes of the lane's token per 64-dim chunk) and V (word j of 8 tokens).
+    // A step is a chain of dependent memory accesses: block id -> row address -> data.  The ids of
+    // all steps in flight are fetched (and waited for) before the first data load, because memory
+    // returns in order and a lookup issued behind another step's data would wait for it; and the
+    // ids of the first round are fetched without waiting for the context length (any token index
+    // below max_ctx is inside the table; entries past the context are replaced below), so that the
+    // length, the query and the ids arrive together instead of one after the other.
+    struct Step {
+        int kid[2], vid[2][FAST ? 1 : 4];
+        int64_t kbase[2], vbase[2][4];
+        u32x4 kw[2][RB];
+        uint32_t vw[RB][2][4];
+    };
+    constexpr int NF = D == 64 ? 4 : (D == 128 ? 2 : 1);
+    Step steps[NF];
+    const int t_cap = max(max_ctx - 1, 0);
+    auto fetch_ids = [&](Step &T, int t0) {
+#pragma unroll
+        for (int a = 0; a < 2; a++) {
+            T.kid[a] = bt[blk_of(min(t0 + 16 * a + j, t_cap))];
+#pragma unroll
+            for (int r = 0; r < (FAST ? 1 : 4); r++) T.vid[a][r] = bt[blk_of(min(t0 + 16 * a + 4 * kb + r, t_cap))];
+        }
+    };
+    int fallback = 0;                             // block of the split's first token: valid whenever the split has work
+    if (max_ctx > 0) {
+        fallback = bt[blk_of(min(t_begin, t_cap))];
+#pragma unroll
+        for (int f = 0; f < NF; f++) fetch_ids(steps[f], t_begin + kStepTok * (wave + kPaWaves * f));
+    }
+
+    const int ctx = min(ctx_raw, max_ctx);        // never index past the block table
     if (t_begin >= ctx) {                         // empty split: the merge never reads it
         if (n_splits == 1) {                      // no merge pass: an empty context gives a zero result
             for (int i = threadIdx.x; i < group * DW; i += kPaThreads) {
@@ -96,23 +144,10 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     }
     const int t_end = min(t_begin + kSplit, ctx);
     const int n_steps = (t_end - t_begin + kStepTok - 1) / kStepTok;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, kb = lane >> 4;
-    auto blk_of = [&](int tok) { return FAST ? tok >> bs_shift : tok / block_size; };
-    auto slot_of = [&](int tok) { return FAST ? tok & (block_size - 1) : tok % block_size; };
 
-    const int32_t *bt = block_tables + (int64_t)seq * max_blocks;
-
-    const int qh = kvh * group + j;  // this lane's query head (valid if j < group)
-    // Q fragments: k-slot mapping of step st: dims 64 (st / 2) + 16 kb + 8 (st % 2) + {0..7}
     half8_t qf[STEPS];
 #pragma unroll
-    for (int st = 0; st < STEPS; st++) {
-        u32x2 w = u32x2{0, 0};
-        if (j < group)
-            w = *reinterpret_cast<const u32x2 *>(q + (int64_t)(seq * n_q_heads + qh) * DW + 16 * (st / 2) + 4 * kb +
-                                                 2 * (st % 2));
-        qf[st] = pa_dec8<MODE>(w.x, w.y);
-    }
+    for (int st = 0; st < STEPS; st++) qf[st] = pa_dec8<MODE>(qw[st].x, qw[st].y);
 
     float4_t o[RB][4];
 #pragma unroll
@@ -121,31 +156,23 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         for (int c = 0; c < 4; c++) o[rb][c] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    // One step = packed K (16 codes of the lane's token per 64-dim chunk) and V (word j of 8 tokens).
-    // Loading is split in two phases so that the table lookups of ALL steps in flight are issued
-    // (and waited for) before the first data load: memory returns in order, so a lookup issued
-    // behind another step's data loads would have to wait for them.
-    struct Step {
-        int64_t kbase[2], vbase[2][4];
-        u32x4 kw[2][RB];
-        uint32_t vw[RB][2][4];
-    };
+    // rows past the context read the fallback block (valid memory) and are masked later
     auto row_base = [&](int blk, int tok) { return ((int64_t)blk * n_kv_heads + kvh) * block_size + slot_of(tok); };
-    auto lookup_step = [&](Step &S, int t0) {
+    auto resolve_step = [&](Step &T, int t0) {
 #pragma unroll
         for (int a = 0; a < 2; a++) {
-            int tc = min(t0 + 16 * a + j, ctx - 1);       // clamp: rows past the context are masked later
-            S.kbase[a] = row_base(bt[blk_of(tc)], tc);
+            const int tk = t0 + 16 * a + j;
+            T.kbase[a] = row_base(tk < ctx ? T.kid[a] : fallback, tk);
             if constexpr (FAST) {
-                int tq = min(t0 + 16 * a + 4 * kb, ctx - 1);
-                int64_t qb = row_base(bt[blk_of(tq)], t0 + 16 * a + 4 * kb);
+                const int tq = t0 + 16 * a + 4 * kb;  // an aligned group of 4 tokens shares a block
+                const int64_t qb = row_base(tq < ctx ? T.vid[a][0] : fallback, tq);
 #pragma unroll
-                for (int r = 0; r < 4; r++) S.vbase[a][r] = qb + r;
+                for (int r = 0; r < 4; r++) T.vbase[a][r] = qb + r;
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    int tv = min(t0 + 16 * a + 4 * kb + r, ctx - 1);
-                    S.vbase[a][r] = row_base(bt[blk_of(tv)], tv);
+                    const int tv = t0 + 16 * a + 4 * kb + r;
+                    T.vbase[a][r] = row_base(tv < ctx ? T.vid[a][r] : fallback, tv);
                 }
             }
         }
@@ -218,22 +245,23 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         }
     };
 
-    {   // The wave's steps are wave, wave + 4, ...  All loads of NF steps are issued before the first
-        // result is needed: a step is a dependent chain (block id -> row address -> data) of several
-        // microseconds, and a wave has only a handful of steps, so they must overlap each other.
-        constexpr int NF = D == 64 ? 4 : (D == 128 ? 2 : 1);
-        Step S[NF];
-        for (int st = wave; st < n_steps; st += kPaWaves * NF) {
+    // The wave's steps are wave, wave + 4, ...; NF of them are in flight together: a wave has only
+    // a handful of steps, so their chains must overlap each other.
+    for (int st = wave; st < n_steps; st += kPaWaves * NF) {
+        if (st != wave) {
 #pragma unroll
             for (int f = 0; f < NF; f++)
-                if (st + kPaWaves * f < n_steps) lookup_step(S[f], t_begin + kStepTok * (st + kPaWaves * f));
-#pragma unroll
-            for (int f = 0; f < NF; f++)
-                if (st + kPaWaves * f < n_steps) load_step(S[f], t_begin + kStepTok * (st + kPaWaves * f));
-#pragma unroll
-            for (int f = 0; f < NF; f++)
-                if (st + kPaWaves * f < n_steps) compute_step(S[f], t_begin + kStepTok * (st + kPaWaves * f));
+                if (st + kPaWaves * f < n_steps) fetch_ids(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
         }
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+            if (st + kPaWaves * f < n_steps) resolve_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+            if (st + kPaWaves * f < n_steps) load_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+            if (st + kPaWaves * f < n_steps) compute_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
     }
 
     // ---- merge the four waves through LDS (wave 0 finishes)

@@ -195,8 +195,7 @@ __global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *
 static int plan_splits(int64_t M, int64_t K) {
     if (K % 256 != 0 || K == 0) return 1;          // the per-vector fallback writes complete sums
     const int64_t tiles = (M + 63) / 64, n_chunks = K / 256;
-    static const int target = getenv("FEATHER_BG_TARGET") ? atoi(getenv("FEATHER_BG_TARGET")) : 256;
-    int64_t s = (target + tiles - 1) / tiles;
+    int64_t s = (256 + tiles - 1) / tiles;       // measured: 128 or 512 workgroups per GEMV are both slower
     s = s < 1 ? 1 : (s > 16 ? 16 : s);
     s = s > n_chunks ? n_chunks : s;
     const int64_t cps = (n_chunks + s - 1) / s;

@@ -77,9 +77,13 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     __shared__ float ml_lds[kPaWaves][2][16];
     __shared__ float4_t o_lds[kPaWaves - 1][RB * 4][kWave];
 
-    const int split = blockIdx.x % n_splits;
-    const int kvh = (blockIdx.x / n_splits) % n_kv_heads;
-    const int seq = blockIdx.x / (n_splits * n_kv_heads);
+    // Consecutive workgroups go to consecutive XCDs.  Split-major order puts the (sequence, head)
+    // pairs of one split on all XCDs alike; with the split index fastest, all first splits (the
+    // ones every sequence has) would land on the same XCD whenever n_splits is a multiple of 8.
+    const int n_pairs = gridDim.x / n_splits;
+    const int split = blockIdx.x / n_pairs;
+    const int kvh = (blockIdx.x % n_pairs) % n_kv_heads;
+    const int seq = (blockIdx.x % n_pairs) / n_kv_heads;
     const int group = n_q_heads / n_kv_heads;
     const int ctx_raw = ctx_lens[seq];
     const int t_begin = split * kSplit;
@@ -108,7 +112,6 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     // length, the query and the ids arrive together instead of one after the other.
     struct Step {
         int kid[2], vid[2][FAST ? 1 : 4];
-        int64_t kbase[2], vbase[2][4];
         u32x4 kw[2][RB];
         uint32_t vw[RB][2][4];
     };
@@ -156,39 +159,27 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         for (int c = 0; c < 4; c++) o[rb][c] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    // rows past the context read the fallback block (valid memory) and are masked later
+    // Row addresses are formed right before the loads (only the block ids of the steps in flight
+    // stay in registers).  Rows past the context read the fallback block (valid memory) and are
+    // masked later.
     auto row_base = [&](int blk, int tok) { return ((int64_t)blk * n_kv_heads + kvh) * block_size + slot_of(tok); };
-    auto resolve_step = [&](Step &T, int t0) {
-#pragma unroll
-        for (int a = 0; a < 2; a++) {
-            const int tk = t0 + 16 * a + j;
-            T.kbase[a] = row_base(tk < ctx ? T.kid[a] : fallback, tk);
-            if constexpr (FAST) {
-                const int tq = t0 + 16 * a + 4 * kb;  // an aligned group of 4 tokens shares a block
-                const int64_t qb = row_base(tq < ctx ? T.vid[a][0] : fallback, tq);
-#pragma unroll
-                for (int r = 0; r < 4; r++) T.vbase[a][r] = qb + r;
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const int tv = t0 + 16 * a + 4 * kb + r;
-                    T.vbase[a][r] = row_base(tv < ctx ? T.vid[a][r] : fallback, tv);
-                }
-            }
-        }
-    };
     auto load_step = [&](Step &S, int t0) {
 #pragma unroll
         for (int a = 0; a < 2; a++) {
-            const uint32_t *kr = k_cache + S.kbase[a] * DW;
+            const int tk = t0 + 16 * a + j;
+            const uint32_t *kr = k_cache + row_base(tk < ctx ? S.kid[a] : fallback, tk) * DW;
 #pragma unroll
             for (int c64 = 0; c64 < RB; c64++) S.kw[a][c64] = *reinterpret_cast<const u32x4 *>(kr + 16 * c64 + 4 * kb);
+            const int tq = t0 + 16 * a + 4 * kb;
+            const uint32_t *vq = nullptr;
+            if constexpr (FAST)                   // an aligned group of 4 tokens shares a block
+                vq = v_cache + row_base(tq < ctx ? S.vid[a][0] : fallback, tq) * DW + j;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                int tok = t0 + 16 * a + 4 * kb + r;
+                const uint32_t *vr = vq + r * DW;
+                if constexpr (!FAST) vr = v_cache + row_base(tq + r < ctx ? S.vid[a][r] : fallback, tq + r) * DW + j;
 #pragma unroll
-                for (int rb = 0; rb < RB; rb++)
-                    S.vw[rb][a][r] = tok < ctx ? v_cache[S.vbase[a][r] * DW + 16 * rb + j] : 0u;
+                for (int rb = 0; rb < RB; rb++) S.vw[rb][a][r] = tq + r < ctx ? vr[16 * rb] : 0u;
             }
         }
     };
@@ -253,9 +244,6 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
             for (int f = 0; f < NF; f++)
                 if (st + kPaWaves * f < n_steps) fetch_ids(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
         }
-#pragma unroll
-        for (int f = 0; f < NF; f++)
-            if (st + kPaWaves * f < n_steps) resolve_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
 #pragma unroll
         for (int f = 0; f < NF; f++)
             if (st + kPaWaves * f < n_steps) load_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));

@@ -133,3 +133,19 @@ def test_pack_full_size_roundtrip_property(dev):
         assert torch.equal(p.view(torch.int32), p2.view(torch.int32))
         err = (y.float() - x.reshape(-1).float()).abs().max().item()
         assert err <= (0.5 if mode == "E5M2" else 0.26)          # half an ulp at |x| < 8
+
+
+@pytest.mark.gpu
+def test_saved_packed_matrix_feeds_gemv_unchanged(dev, tmp_path):
+    import feather_amd as feather
+    from feather_amd.packers.serial import PackedTensor, load_packed, save_packed
+    g = torch.Generator(device=dev).manual_seed(11)
+    m = torch.randn(96, 256, generator=g, device=dev).half()
+    v = torch.randn(256, generator=g, device=dev).half()
+    mp, vp = feather.pack_fp8_tensor(m, mode="E4M3"), feather.pack_fp8_tensor(v, mode="E4M3")
+    save_packed(tmp_path / "m.fthr", PackedTensor(mp, m.shape, "E4M3"))
+    back = load_packed(tmp_path / "m.fthr", device=dev)
+    assert back.shape == (96, 256) and back.words.device == mp.device
+    assert torch.equal(back.words.view(torch.int32), mp.view(torch.int32))
+    assert torch.equal(feather.gemv(back.words, vp, original_shape=back.shape, mode=back.mode),
+                       feather.gemv(mp, vp, original_shape=m.shape, mode="E4M3"))

@@ -39,6 +39,10 @@ SIGNATURES = {
     "feather_dot_fp8": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _vp]),
     "feather_dot_fp16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _vp]),
     "feather_flash_attn_fp8": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _f32, _i32, _vp]),
+    "feather_flash_attn_fp8_varlen": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _f32,
+                                             _i32, _vp]),
+    "feather_paged_cache_write": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
+                                         _i32, _vp]),
     "feather_paged_attn_scratch_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "feather_paged_attn_fp8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                       _i32, _f32, _vp]),

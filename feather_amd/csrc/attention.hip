@@ -1,4 +1,5 @@
-// Non-causal flash-attention forward on FP8-packed Q/K/V (prefill).
+// Flash-attention forward on FP8-packed Q/K/V (prefill): fixed-length heads, or variable-length
+// sequences packed back to back with an optional causal mask.
 //
 // Work split.  One workgroup (4 waves) owns a tile of 64*QB queries of one
 // head; each wave owns 16*QB of them for the whole key loop.  Keys/values are
@@ -58,11 +59,16 @@ __device__ __forceinline__ float xor_lane(float x, int mask) {
 // BN  keys per tile
 // OCC workgroups per CU the register budget is sized for (2 keeps every MFMA
 //     accumulator in architectural VGPRs, so rescaling needs no AGPR copies)
-template <int D, int MODE, int QB, int SB, int BN, int OCC>
+// VC  variable-length / causal variant: every head holds total_rows rows, sequence s of
+//     cu_seqlens (n_seq + 1 row offsets) occupies rows [cu[s], cu[s+1]) of every head and
+//     attends only to itself; with causal != 0 query i sees keys 0..i of its sequence.
+//     tiles_per_head = n_seq * tiles_per_seq; L, keys_scored and mask_tail are not used.
+template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC>
 __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
     const uint32_t *__restrict__ q, const uint32_t *__restrict__ k, const uint32_t *__restrict__ v,
     float *__restrict__ out, int L, int n_heads, int kv_group, int tiles_per_head, float scale_log2e,
-    int keys_scored, int mask_tail) {
+    int keys_scored, int mask_tail, const int32_t *__restrict__ cu_seqlens, int tiles_per_seq, int total_rows,
+    int causal) {
     constexpr int DW = D / 4;              // packed words per row
     constexpr int KS = D + 8;              // fp16 per K row in LDS (16 B pad against bank conflicts)
     constexpr int VS = BN;                 // fp16 per V^T row in LDS (16-byte chunks XOR-swizzled by row)
@@ -88,16 +94,30 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
     const int total = gridDim.x;
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
     const int head = bid / tiles_per_head;
-    const int tile = bid % tiles_per_head;
+    int tile = bid % tiles_per_head;
     const int kv_head = head / kv_group;
+    int64_t q_row0 = (int64_t)head * L, kv_row0 = (int64_t)kv_head * L;   // first row of this head's sequence
+    if constexpr (VC) {
+        const int seq = tile / tiles_per_seq;
+        tile = tile % tiles_per_seq;
+        if (causal) tile = tiles_per_seq - 1 - tile;          // the tiles with the longest key loops start first
+        const int r0 = cu_seqlens[seq];
+        L = cu_seqlens[seq + 1] - r0;
+        if (tile * (64 * QB) >= L) return;                    // past the end of this sequence (whole workgroup)
+        q_row0 = (int64_t)head * total_rows + r0;
+        kv_row0 = (int64_t)kv_head * total_rows + r0;
+        mask_tail = 1;
+        const int last_key = causal ? min(L, (tile + 1) * (64 * QB)) : L;
+        keys_scored = (last_key + BN - 1) / BN * BN;
+    }
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 15, kb = lane >> 4;
     const int q0 = tile * QT + wave * (16 * QB);
 
-    const uint32_t *qh = q + (int64_t)head * L * DW;
-    const uint32_t *kh = k + (int64_t)kv_head * L * DW;
-    const uint32_t *vh = v + (int64_t)kv_head * L * DW;
+    const uint32_t *qh = q + q_row0 * DW;
+    const uint32_t *kh = k + kv_row0 * DW;
+    const uint32_t *vh = v + kv_row0 * DW;
 
     // ---- Q fragments (B operand of S^T), resident in registers
     half8_t qf[QB][STEPS];
@@ -205,6 +225,12 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
         const _Float16 *k_lds = lds + cur * kBufHalfs;
         const _Float16 *vt_lds = k_lds + BN * KS;
         const bool ragged = mask_tail && key0 + BN > L;   // only the last tile can hold masked keys
+        bool diag = false, skip = false;
+        if constexpr (VC) {
+            diag = causal && key0 + BN - 1 > q0;          // some key of the tile lies past the wave's first query
+            skip = causal && key0 > q0 + 16 * QB - 1;     // every key lies past the wave's last query
+        }
+        if (!skip) {
 
         half8_t pf[QB][KB32];
         // query blocks are scored SB at a time: the K fragments are re-used across the SB
@@ -228,12 +254,13 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
             // p = 2^(s * c - m * c).
 #pragma unroll
             for (int b = 0; b < SB; b++) {
-                if (ragged) {
+                if (ragged || diag) {
+                    const int last = diag ? min(L - 1, q0 + 16 * (b0 + b) + j) : L - 1;   // last visible key
 #pragma unroll
                     for (int c = 0; c < KB16; c++)
 #pragma unroll
                         for (int r = 0; r < 4; r++)
-                            if (key0 + 16 * c + 4 * kb + r >= L) s[b][c][r] = -INFINITY;
+                            if (key0 + 16 * c + 4 * kb + r > last) s[b][c][r] = -INFINITY;
                 }
                 float mx = s[b][0][0];
 #pragma unroll
@@ -280,11 +307,12 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
 #pragma unroll
             for (int b = 0; b < QB; b++) o[b][DB] = mfma16(ones, pf[b][t], o[b][DB]);
         }
+        }   // !skip
         __syncthreads();  // tile i+1 is visible; every wave is done reading tile i
     }
 
     // ---- epilogue: finish the row sums, normalise, store [q][dd]
-    float *oh = out + (int64_t)head * L * D;
+    float *oh = out + q_row0 * D;
 #pragma unroll
     for (int b = 0; b < QB; b++) {
         const float l = o[b][DB][0];   // row 4 * kb of the ones block: the full sum over keys
@@ -298,17 +326,32 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
     }
 }
 
-template <int D, int MODE, int QB, int SB, int BN, int OCC>
-static int launch_attn(const void *q, const void *k, const void *v, void *out, int64_t n_heads, int64_t L,
-                       int64_t kv_group, float scale, int tail, hipStream_t s) {
+// Fixed-length heads (cu_seqlens == nullptr; L rows per head) or packed variable-length sequences
+// (cu_seqlens given: n_seq sequences of at most max_seqlen rows inside total_rows rows per head).
+struct AttnArgs {
+    const void *q, *k, *v;
+    void *out;
+    int64_t n_heads, L, kv_group;
+    float scale;
+    int tail;
+    const void *cu_seqlens;
+    int64_t n_seq, max_seqlen, total_rows;
+    int causal;
+};
+
+template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC>
+static int launch_attn(const AttnArgs &a, hipStream_t s) {
     constexpr int QT = 64 * QB;
     constexpr size_t lds = (size_t)(BN * (D + 8) + D * BN) * 2 * 2;  // two (K, V^T) buffers
-    int tiles = (int)((L + QT - 1) / QT);
-    int64_t blocks = tiles * n_heads;
+    const int64_t L = VC ? a.max_seqlen : a.L;
+    const int tiles_per_seq = (int)((L + QT - 1) / QT);
+    const int64_t tiles = VC ? tiles_per_seq * a.n_seq : tiles_per_seq;
+    const int64_t blocks = tiles * a.n_heads;
     FEATHER_CHECK(blocks < (1ll << 31), FEATHER_ESHAPE, "feather_flash_attn_fp8: grid too large");
+    if (blocks == 0) return FEATHER_OK;
     // the reference scores whole 64-key tiles (zero rows past L); otherwise only tiles of BN up to L
-    int64_t keys_scored = tail == FEATHER_TAIL_REFERENCE ? (L + 63) / 64 * 64 : (L + BN - 1) / BN * BN;
-    auto kern = flash_attn_kernel<D, MODE, QB, SB, BN, OCC>;
+    int64_t keys_scored = a.tail == FEATHER_TAIL_REFERENCE ? (L + 63) / 64 * 64 : (L + BN - 1) / BN * BN;
+    auto kern = flash_attn_kernel<D, MODE, QB, SB, BN, OCC, VC>;
     if (lds > 64 * 1024) {
         static bool attr_set = false;  // per instantiation
         if (!attr_set) {
@@ -320,20 +363,21 @@ static int launch_attn(const void *q, const void *k, const void *v, void *out, i
         }
     }
     const float log2e = 1.4426950408889634f;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kAttnThreads), lds, s, (const uint32_t *)q,
-                       (const uint32_t *)k, (const uint32_t *)v, (float *)out, (int)L, (int)n_heads, (int)kv_group,
-                       tiles, scale * log2e, (int)keys_scored, tail == FEATHER_TAIL_MASK ? 1 : 0);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kAttnThreads), lds, s, (const uint32_t *)a.q,
+                       (const uint32_t *)a.k, (const uint32_t *)a.v, (float *)a.out, (int)L, (int)a.n_heads,
+                       (int)a.kv_group, (int)tiles, a.scale * log2e, (int)keys_scored,
+                       a.tail == FEATHER_TAIL_MASK ? 1 : 0, (const int32_t *)a.cu_seqlens, tiles_per_seq,
+                       (int)a.total_rows, a.causal);
     return check_launch("feather_flash_attn_fp8");
 }
 
-template <int MODE>
-static int dispatch_attn(const void *q, const void *k, const void *v, void *out, int64_t n_heads, int64_t L, int64_t d,
-                         int64_t kv_group, float scale, int tail, hipStream_t s) {
+template <int MODE, bool VC>
+static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
     switch (d) {
-        case 64: return launch_attn<64, MODE, 4, 2, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-        case 128: return launch_attn<128, MODE, 2, 2, 64, 2>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-        case 256: return launch_attn<256, MODE, 1, 1, 32, 1>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
-        case 512: return launch_attn<512, MODE, 1, 1, 32, 1>(q, k, v, out, n_heads, L, kv_group, scale, tail, s);
+        case 64: return launch_attn<64, MODE, 4, 2, 64, 2, VC>(a, s);
+        case 128: return launch_attn<128, MODE, 2, 2, 64, 2, VC>(a, s);
+        case 256: return launch_attn<256, MODE, 1, 1, 32, 1, VC>(a, s);
+        case 512: return launch_attn<512, MODE, 1, 1, 32, 1, VC>(a, s);
     }
     set_error("feather_flash_attn_fp8: head dim %lld not supported (64, 128, 256, 512)", (long long)d);
     return FEATHER_ESHAPE;
@@ -360,6 +404,34 @@ extern "C" int feather_flash_attn_fp8(const void *q, const void *k, const void *
     FEATHER_CHECK(aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out_f32, 16), FEATHER_EINVAL,
                   "feather_flash_attn_fp8: pointers must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
-    if (mode == FEATHER_E5M2) return dispatch_attn<FEATHER_E5M2>(q, k, v, out_f32, n_heads, L, d, kv_group, scale, tail, s);
-    return dispatch_attn<FEATHER_E4M3>(q, k, v, out_f32, n_heads, L, d, kv_group, scale, tail, s);
+    const AttnArgs a = {q, k, v, out_f32, n_heads, L, kv_group, scale, tail, nullptr, 0, 0, 0, 0};
+    if (mode == FEATHER_E5M2) return dispatch_attn<FEATHER_E5M2, false>(a, d, s);
+    return dispatch_attn<FEATHER_E4M3, false>(a, d, s);
+}
+
+extern "C" int feather_flash_attn_fp8_varlen(const void *q, const void *k, const void *v, void *out_f32,
+                                             const void *cu_seqlens, int64_t n_seq, int64_t max_seqlen,
+                                             int64_t total_rows, int64_t n_heads, int64_t d, int64_t kv_group, int mode,
+                                             float scale, int causal, void *stream) {
+    const char *me = "feather_flash_attn_fp8_varlen";
+    FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE, "%s: mode %d not supported", me, mode);
+    FEATHER_CHECK(n_heads >= 0 && n_seq >= 0 && max_seqlen >= 0 && total_rows >= 0 && d > 0, FEATHER_EINVAL,
+                  "%s: negative shape", me);
+    FEATHER_CHECK(causal == 0 || causal == 1, FEATHER_EINVAL, "%s: causal must be 0 or 1", me);
+    FEATHER_CHECK(kv_group >= 1 && n_heads % kv_group == 0, FEATHER_ESHAPE,
+                  "%s: n_heads=%lld is not a multiple of kv_group=%lld", me, (long long)n_heads, (long long)kv_group);
+    FEATHER_CHECK(max_seqlen <= total_rows && total_rows < (1ll << 30), FEATHER_ESHAPE,
+                  "%s: max_seqlen=%lld must not exceed total_rows=%lld (< 2^30)", me, (long long)max_seqlen,
+                  (long long)total_rows);
+    FEATHER_CHECK(d == 64 || d == 128 || d == 256 || d == 512, FEATHER_ESHAPE,
+                  "%s: head dim %lld not supported (64, 128, 256, 512)", me, (long long)d);
+    if (n_heads == 0 || n_seq == 0 || max_seqlen == 0) return FEATHER_OK;
+    FEATHER_CHECK(q && k && v && out_f32 && cu_seqlens, FEATHER_EINVAL, "%s: null pointer", me);
+    FEATHER_CHECK(aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out_f32, 16) && aligned(cu_seqlens, 4),
+                  FEATHER_EINVAL, "%s: q/k/v/out must be 16-byte aligned", me);
+    hipStream_t s = (hipStream_t)stream;
+    const AttnArgs a = {q, k, v, out_f32, n_heads, 0, kv_group, scale, FEATHER_TAIL_MASK, cu_seqlens, n_seq,
+                        max_seqlen, total_rows, causal};
+    if (mode == FEATHER_E5M2) return dispatch_attn<FEATHER_E5M2, true>(a, d, s);
+    return dispatch_attn<FEATHER_E4M3, true>(a, d, s);
 }

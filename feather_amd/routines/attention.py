@@ -16,15 +16,16 @@ import torch
 from .. import _native as N
 
 __all__ = ["flash_attention_fp8_e5m2_acc_fp32_gpu", "flash_attention_fp8_e4m3_acc_fp32_gpu",
-           "flash_attention_fp8_acc_fp32_gpu"]
+           "flash_attention_fp8_acc_fp32_gpu", "flash_attention_fp8_varlen_acc_fp32_gpu"]
 
 _TAILS = {"mask": N.TAIL_MASK, "reference": N.TAIL_REFERENCE}
 
 
 def flash_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seq_len: int, h_dim: int, *,
                                      mode: str = "E5M2", scale: float | None = None, tail: str = "mask",
-                                     kv_group: int = 1) -> torch.Tensor:
-    """``softmax(Q K^T * scale) V`` per head, non-causal.
+                                     kv_group: int = 1, causal: bool = False) -> torch.Tensor:
+    """``softmax(Q K^T * scale) V`` per head; non-causal unless ``causal=True``
+    (query ``i`` then sees keys ``0..i``; needs ``tail="mask"``).
 
     ``q`` holds ``n_heads * seq_len * h_dim`` packed words (``h_dim = d // 4``);
     ``k``/``v`` hold ``n_heads // kv_group`` heads.  Returns float32
@@ -56,7 +57,13 @@ def flash_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: torch.
     if scale is None:
         scale = 1.0 / math.sqrt(d)
     out = torch.empty((n_heads, seq_len, d), dtype=torch.float32, device=q.device)
-    N.call(q.device, "feather_flash_attn_fp8", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), n_heads, seq_len, d, kv_group, code, float(scale), _TAILS[tail])
+    if causal:
+        if tail != "mask":
+            raise ValueError("causal attention needs tail='mask'")
+        cu = torch.tensor([0, seq_len], dtype=torch.int32, device=q.device)
+        N.call(q.device, "feather_flash_attn_fp8_varlen", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(cu), 1, seq_len, seq_len, n_heads, d, kv_group, code, float(scale), 1)
+    else:
+        N.call(q.device, "feather_flash_attn_fp8", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), n_heads, seq_len, d, kv_group, code, float(scale), _TAILS[tail])
     if q.dim() >= 2 and q.shape[-2:] == (seq_len, h_dim):
         return out.view(*q.shape[:-2], seq_len, d)
     return out[0] if n_heads == 1 else out
@@ -78,3 +85,38 @@ def flash_attention_fp8_e4m3_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: t
     (gemv.py:83-88)."""
     return flash_attention_fp8_acc_fp32_gpu(q, k, v, seq_len, h_dim, mode="E4M3", scale=scale, tail=tail,
                                             kv_group=kv_group)
+
+
+def flash_attention_fp8_varlen_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor,
+                                            max_seqlen: int, *, mode: str = "E5M2", scale: float | None = None,
+                                            causal: bool = False) -> torch.Tensor:
+    """Attention over variable-length sequences packed back to back (no counterpart in
+    the reference).
+
+    q            ``[n_heads, total_rows, d/4]`` packed words
+    k, v         ``[n_kv_heads, total_rows, d/4]`` (query head ``h`` reads KV head ``h // (n_heads // n_kv_heads)``)
+    cu_seqlens   ``[n_seq + 1]`` int32 on the device: sequence ``s`` is rows ``cu[s] .. cu[s+1]-1``
+    max_seqlen   upper bound of the sequence lengths (sizes the grid, no device-to-host copy)
+    Returns float32 ``[n_heads, total_rows, d]``; rows outside every sequence are zero."""
+    code = N.mode_code(mode)
+    q, k, v = N.as_words(q, "q"), N.as_words(k, "k"), N.as_words(v, "v")
+    if q.dim() != 3 or k.dim() != 3 or v.shape != k.shape or k.shape[1:] != q.shape[1:]:
+        raise ValueError("expected q [n_heads, total_rows, d/4] and k, v [n_kv_heads, total_rows, d/4]")
+    n_heads, total, dw = q.shape
+    n_kv = k.shape[0]
+    d = 4 * dw
+    if d not in (64, 128, 256, 512):
+        raise ValueError(f"head dim {d} not supported: 64, 128, 256 or 512")
+    if n_kv == 0 or n_heads % n_kv != 0:
+        raise ValueError(f"n_heads={n_heads} is not a multiple of n_kv_heads={n_kv}")
+    if cu_seqlens.dtype != torch.int32 or cu_seqlens.dim() != 1 or cu_seqlens.numel() < 1 or not cu_seqlens.is_cuda:
+        raise ValueError("cu_seqlens must be a 1-D int32 tensor of n_seq + 1 offsets on the device")
+    max_seqlen = int(max_seqlen)
+    if max_seqlen < 0 or max_seqlen > total:
+        raise ValueError(f"max_seqlen={max_seqlen} outside [0, total_rows={total}]")
+    if scale is None:
+        scale = 1.0 / math.sqrt(d)
+    out = torch.zeros((n_heads, total, d), dtype=torch.float32, device=q.device)
+    cu_seqlens = cu_seqlens.contiguous()
+    N.call(q.device, "feather_flash_attn_fp8_varlen", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(cu_seqlens), cu_seqlens.numel() - 1, max_seqlen, total, n_heads, d, n_heads // n_kv, code, float(scale), 1 if causal else 0)
+    return out

@@ -11,7 +11,7 @@ import torch
 
 from .. import _native as N
 
-__all__ = ["paged_attention_fp8_acc_fp32_gpu"]
+__all__ = ["paged_attention_fp8_acc_fp32_gpu", "paged_cache_write"]
 
 
 def paged_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -57,3 +57,48 @@ def paged_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k_cache: torch.Tensor, v_c
     scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
     N.call(q.device, "feather_paged_attn_fp8", N.ptr(q), N.ptr(k_cache), N.ptr(v_cache), N.ptr(block_tables), N.ptr(context_lens), N.ptr(out), N.ptr(scratch), n_seq, n_q_heads, n_kv_heads, d, block_size, max_blocks, max_ctx, code, float(scale))
     return out
+
+
+def paged_cache_write(k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      block_tables: torch.Tensor, cu_seqlens: torch.Tensor, start_pos: torch.Tensor | None = None, *,
+                      mode: str = "E5M2") -> None:
+    """Write the K and V rows of packed variable-length sequences into a paged cache, in place.
+
+    k, v          ``[n_kv_heads, total_rows, d/4]`` packed words, or ``[n_kv_heads, total_rows, d]`` float16
+                  (then encoded to ``mode`` on the device, as ``pack_fp8_tensor``)
+    k_cache       ``[n_blocks, n_kv_heads, block_size, d/4]`` packed words (``v_cache`` alike)
+    block_tables  ``[n_seq, max_blocks]`` int32; ``cu_seqlens`` ``[n_seq + 1]`` int32
+    start_pos     ``[n_seq]`` int32 cache position of each sequence's first row (default 0)
+    Row ``cu[s] + i`` lands at position ``start_pos[s] + i`` of sequence ``s``; positions past the block
+    table are dropped."""
+    code = N.mode_code(mode)
+    k_cache, v_cache = N.as_words(k_cache, "k_cache"), N.as_words(v_cache, "v_cache")
+    if k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
+        raise ValueError("expected k_cache/v_cache [n_blocks, n_kv_heads, block_size, d/4]")
+    n_blocks, n_kv, block_size, dw = k_cache.shape
+    d = 4 * dw
+    f16 = k.dtype == torch.float16
+    if f16:
+        if v.dtype != torch.float16:
+            raise ValueError("k and v must both be float16 or both packed words")
+        k, v = k.contiguous(), v.contiguous()
+        want = (n_kv, k.shape[1] if k.dim() == 3 else -1, d)
+    else:
+        k, v = N.as_words(k, "k"), N.as_words(v, "v")
+        want = (n_kv, k.shape[1] if k.dim() == 3 else -1, dw)
+    if k.dim() != 3 or tuple(k.shape) != want or v.shape != k.shape:
+        raise ValueError(f"expected k and v of shape [n_kv_heads={n_kv}, total_rows, {want[2]}], got {tuple(k.shape)} and {tuple(v.shape)}")
+    if d % 16 != 0:
+        raise ValueError(f"head dim {d} is not a multiple of 16")
+    total = k.shape[1]
+    for name, t in (("block_tables", block_tables), ("cu_seqlens", cu_seqlens), ("start_pos", start_pos)):
+        if t is not None and (t.dtype != torch.int32 or not t.is_cuda):
+            raise ValueError(f"{name} must be an int32 tensor on the device")
+    n_seq = cu_seqlens.numel() - 1
+    if cu_seqlens.dim() != 1 or n_seq < 0 or block_tables.dim() != 2 or block_tables.shape[0] != n_seq:
+        raise ValueError("cu_seqlens must be [n_seq + 1] and block_tables [n_seq, max_blocks]")
+    if start_pos is not None and start_pos.shape != (n_seq,):
+        raise ValueError("start_pos must be [n_seq]")
+    block_tables, cu_seqlens = block_tables.contiguous(), cu_seqlens.contiguous()
+    sp = N.ptr(start_pos.contiguous()) if start_pos is not None else None
+    N.call(k.device, "feather_paged_cache_write", N.ptr(k), N.ptr(v), 1 if f16 else 0, N.ptr(k_cache), N.ptr(v_cache), N.ptr(block_tables), N.ptr(cu_seqlens), sp, n_seq, total, n_kv, d, block_size, block_tables.shape[1], code)

@@ -115,7 +115,7 @@ int feather_dot_fp8(const void *x1, const void *x2, void *out_f32, void *scratch
 int feather_dot_fp16(const void *x1, const void *x2, void *out_f32, void *scratch, int64_t n_words, int fp16_products,
                      void *stream);
 
-/* Non-causal attention forward on packed Q/K/V: for each of n_heads
+/* Non-causal attention forward on packed Q/K/V of fixed length: for each of n_heads
  * independent heads, out[h] = softmax(Q K^T * scale) V, Q/K/V [L, d/4] words,
  * out [L, d] fp32; scores fp32, P rounded to fp16 before P.V, fp32 output.
  * d in {64, 128, 256, 512}.  kv_group > 1 maps query head h to K/V head
@@ -125,6 +125,35 @@ int feather_dot_fp16(const void *x1, const void *x2, void *out_f32, void *scratc
  * scale = 1/sqrt(d), tail = REFERENCE. */
 int feather_flash_attn_fp8(const void *q, const void *k, const void *v, void *out_f32, int64_t n_heads, int64_t L,
                            int64_t d, int64_t kv_group, int mode, float scale, int tail, void *stream);
+
+/* Attention forward on packed variable-length sequences, optionally causal.  No reference
+ * counterpart (the reference kernel, feather/routines/attention.py:14-108, is one
+ * fixed-length non-causal head); numerics as feather_flash_attn_fp8 with the exact tail.
+ *   q            [n_heads, total_rows, d/4] words; k, v [n_heads / kv_group, total_rows, d/4]
+ *   cu_seqlens   [n_seq + 1] int32 on the device, non-decreasing row offsets: sequence s is
+ *                rows cu[s] .. cu[s+1]-1 of every head and attends only to itself
+ *   max_seqlen   upper bound of cu[s+1] - cu[s] (sizes the grid; rows past it are not computed)
+ *   out          [n_heads, total_rows, d] fp32; rows outside every sequence are left untouched
+ *   causal       1: query i of a sequence sees keys 0..i of that sequence
+ * A fixed-length batch is n_seq = 1, cu = {0, L}, n_heads = batch * heads. */
+int feather_flash_attn_fp8_varlen(const void *q, const void *k, const void *v, void *out_f32, const void *cu_seqlens,
+                                  int64_t n_seq, int64_t max_seqlen, int64_t total_rows, int64_t n_heads, int64_t d,
+                                  int64_t kv_group, int mode, float scale, int causal, void *stream);
+
+/* Scatter the K and V rows of packed variable-length sequences (the layout of
+ * feather_flash_attn_fp8_varlen) into a paged cache.  No reference counterpart.
+ *   k_src, v_src  src_f16 = 0: packed words [n_kv_heads, total_rows, d/4];
+ *                 src_f16 = 1: fp16 [n_kv_heads, total_rows, d], encoded to `mode` on the way
+ *                 (round to nearest even, as feather_pack_fp8)
+ *   k_cache       [n_blocks, n_kv_heads, block_size, d/4] words (v_cache same)
+ *   block_tables  [n_seq, max_blocks] int32; cu_seqlens [n_seq + 1] int32
+ *   start_pos     [n_seq] int32 or NULL (all 0): cache position of each sequence's first row
+ * Row cu[s] + i goes to position start_pos[s] + i of sequence s.  Positions at or beyond
+ * max_blocks * block_size have no table entry and are dropped.  d % 16 == 0. */
+int feather_paged_cache_write(const void *k_src, const void *v_src, int src_f16, void *k_cache, void *v_cache,
+                              const void *block_tables, const void *cu_seqlens, const void *start_pos, int64_t n_seq,
+                              int64_t total_rows, int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
+                              int mode, void *stream);
 
 /* Bytes of scratch feather_paged_attn_fp8 needs for the given problem. */
 int64_t feather_paged_attn_scratch_bytes(int64_t n_seq, int64_t n_q_heads, int64_t d, int64_t max_ctx);

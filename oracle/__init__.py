@@ -263,3 +263,49 @@ def attention_f64_np(q, k, v, L: int, d: int, mode="E5M2", scale=None) -> np.nda
         P = np.exp(S)
         out[h] = (P @ Vd[h]) / P.sum(axis=1, keepdims=True)
     return out
+
+
+def attention_varlen_f64_np(q, k, v, cu_seqlens, d: int, mode="E5M2", scale=None, causal: bool = False) -> np.ndarray:
+    """Variable-length attention in float64 (closed form): q words [n_heads, total, d/4], k/v words
+    [n_kv_heads, total, d/4]; sequence s is rows cu[s]..cu[s+1]-1 and attends only to itself; with
+    `causal`, query i of a sequence sees keys 0..i.  Rows outside every sequence stay zero."""
+    q, k, v = (np.asarray(a) for a in (q, k, v))
+    n_heads, total = q.shape[0], q.shape[1]
+    n_kv = k.shape[0]
+    group = n_heads // n_kv
+    Q = decode_np(q.reshape(-1), mode).reshape(n_heads, total, d)
+    Kd = decode_np(k.reshape(-1), mode).reshape(n_kv, total, d)
+    Vd = decode_np(v.reshape(-1), mode).reshape(n_kv, total, d)
+    if scale is None:
+        scale = 1.0 / np.sqrt(d)
+    out = np.zeros((n_heads, total, d), dtype=np.float64)
+    cu = [int(c) for c in cu_seqlens]
+    for h in range(n_heads):
+        for a, b in zip(cu[:-1], cu[1:]):
+            if b <= a:
+                continue
+            S = (Q[h, a:b] @ Kd[h // group, a:b].T) * scale
+            if causal:
+                S = np.where(np.tril(np.ones((b - a, b - a), dtype=bool)), S, -np.inf)
+            S = S - S.max(axis=1, keepdims=True)
+            P = np.exp(S)
+            out[h, a:b] = (P @ Vd[h // group, a:b]) / P.sum(axis=1, keepdims=True)
+    return out
+
+
+def paged_cache_write_np(k_words, v_words, k_cache, v_cache, block_tables, cu_seqlens, start_pos=None) -> None:
+    """Scatter packed rows [n_kv_heads, total, d/4] into caches [n_blocks, n_kv_heads, block_size, d/4]
+    in place: row cu[s] + i goes to position start_pos[s] + i of sequence s; positions without a
+    block-table entry are dropped."""
+    n_seq = len(cu_seqlens) - 1
+    block_size, max_blocks = k_cache.shape[2], block_tables.shape[1]
+    for s in range(n_seq):
+        p0 = 0 if start_pos is None else int(start_pos[s])
+        for i, t in enumerate(range(int(cu_seqlens[s]), int(cu_seqlens[s + 1]))):
+            pos = p0 + i
+            if pos < 0 or pos >= max_blocks * block_size:
+                continue
+            blk = int(block_tables[s, pos // block_size])
+            k_cache[blk, :, pos % block_size, :] = k_words[:, t, :]
+            v_cache[blk, :, pos % block_size, :] = v_words[:, t, :]
+

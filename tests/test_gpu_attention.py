@@ -168,3 +168,99 @@ def test_paged_attention_config_shape(dev, orc):
     want = orc.paged_attn(to_np(q).reshape(n_seq, -1)[seqs], to_np(kc), to_np(vc), bt.numpy()[seqs], ctx.numpy()[seqs],
                           Hq, Hkv, d, bs, "E4M3")
     assert _nerr(out.cpu().numpy()[seqs], want) <= TOL
+
+
+# ---------------------------------------------------------------- variable length, causal, cache writer
+
+@pytest.mark.parametrize("mode,n_heads,n_kv,d,lens,causal", [
+    ("E5M2", 2, 1, 64, [70, 0, 300, 1], True), ("E5M2", 2, 2, 64, [70, 0, 300, 1], False),
+    ("E4M3", 4, 2, 64, [513, 255], True), ("E5M2", 1, 1, 128, [129, 64], True),
+    ("E4M3", 1, 1, 256, [100, 37], True), ("E5M2", 1, 1, 512, [65], True), ("E4M3", 2, 1, 128, [200], False),
+])
+def test_varlen_attention_vs_oracle(dev, orc, mode, n_heads, n_kv, d, lens, causal):
+    from feather_amd.routines.attention import flash_attention_fp8_varlen_acc_fp32_gpu
+    rng = np.random.default_rng(sum(lens) + d + n_heads)
+    gap = 3                                                  # rows in front of the first sequence belong to no one
+    cu = np.concatenate([[gap], gap + np.cumsum(lens)]).astype(np.int32)
+    total = int(cu[-1]) + 2
+    q = orc.pack_fp8(rng.standard_normal((n_heads, total, d)).astype(np.float16), mode).reshape(n_heads, total, d // 4)
+    k = orc.pack_fp8(rng.standard_normal((n_kv, total, d)).astype(np.float16), mode).reshape(n_kv, total, d // 4)
+    v = orc.pack_fp8(rng.standard_normal((n_kv, total, d)).astype(np.float16), mode).reshape(n_kv, total, d // 4)
+    out = flash_attention_fp8_varlen_acc_fp32_gpu(_dev_words(q, dev, q.shape), _dev_words(k, dev, k.shape),
+                                                  _dev_words(v, dev, v.shape), torch.from_numpy(cu).to(dev), max(lens),
+                                                  mode=mode, causal=causal).cpu().numpy()
+    want = orc.attention_varlen_f64_np(q, k, v, cu, d, mode, causal=causal)
+    assert _nerr(out, want) <= TOL
+    assert not out[:, :gap].any() and not out[:, int(cu[-1]):].any()      # rows outside every sequence untouched
+
+
+@pytest.mark.parametrize("mode", ["E5M2", "E4M3"])
+def test_causal_fixed_length_rows_equal_prefix_attention(dev, orc, mode):
+    """causal=True of the fixed-length entry: row i equals the non-causal kernel run on keys 0..i
+    (L = 1000: ragged last tile, several query tiles)."""
+    from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
+    rng = np.random.default_rng(21)
+    heads, L, d = 2, 1000, 64
+    q, k, v = _qkv(rng, heads, L, d, mode, orc)
+    qd, kd, vd = (_dev_words(a, dev, (heads, L, d // 4)) for a in (q, k, v))
+    caus = flash_attention_fp8_acc_fp32_gpu(qd, kd, vd, L, d // 4, mode=mode, causal=True)
+    assert caus.shape == (heads, L, d)
+    for i in (0, 63, 64, 255, 256, 700, 999):
+        pre = flash_attention_fp8_acc_fp32_gpu(qd[:, i:i + 1].expand(heads, i + 1, d // 4).contiguous(),
+                                               kd[:, :i + 1].contiguous(), vd[:, :i + 1].contiguous(), i + 1, d // 4, mode=mode)
+        err = (caus[:, i] - pre[:, 0]).abs().max() / pre[:, 0].abs().max()
+        assert err.item() <= TOL
+    with pytest.raises(ValueError):
+        flash_attention_fp8_acc_fp32_gpu(qd, kd, vd, L, d // 4, mode=mode, causal=True, tail="reference")
+
+
+@pytest.mark.parametrize("mode,f16", [("E5M2", False), ("E4M3", False), ("E4M3", True), ("E5M2", True)])
+def test_paged_cache_write_bit_exact(dev, orc, mode, f16):
+    from feather_amd.routines.paged_attention import paged_cache_write
+    rng = np.random.default_rng(8)
+    n_kv, d, bs, max_blocks = 2, 64, 16, 6
+    lens, start = [40, 0, 77, 5], np.array([3, 0, 30, 95], dtype=np.int32)   # sequence 2 overruns 96 slots: rows dropped
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    total, n_blocks = int(cu[-1]) + 4, 4 * max_blocks + 1
+    bt = rng.permutation(n_blocks - 1)[:4 * max_blocks].reshape(4, max_blocks).astype(np.int32)
+    k16, v16 = (rng.standard_normal((n_kv, total, d)).astype(np.float16) * 20 for _ in range(2))
+    k16[0, 1, :4] = [np.inf, -np.inf, 500.0, 1e-4]                            # saturating and tiny values through the encoder
+    kw, vw = (orc.pack_fp8(a, mode).reshape(n_kv, total, d // 4) for a in (k16, v16))
+    fill = rng.integers(0, 2**32, (n_blocks, n_kv, bs, d // 4), dtype=np.uint64).astype(np.uint32)
+    kc, vc = fill.copy(), fill[::-1].copy()
+    kcd, vcd = _dev_words(kc, dev, kc.shape), _dev_words(vc, dev, vc.shape)
+    src = (torch.from_numpy(k16).to(dev), torch.from_numpy(v16).to(dev)) if f16 else \
+        (_dev_words(kw, dev, kw.shape), _dev_words(vw, dev, vw.shape))
+    paged_cache_write(src[0], src[1], kcd, vcd, torch.from_numpy(bt).to(dev), torch.from_numpy(cu).to(dev),
+                      torch.from_numpy(start).to(dev), mode=mode)
+    orc.paged_cache_write_np(kw, vw, kc, vc, bt, cu, start)
+    assert np.array_equal(kcd.cpu().view(torch.int32).numpy().view(np.uint32), kc)      # untouched slots keep their fill
+    assert np.array_equal(vcd.cpu().view(torch.int32).numpy().view(np.uint32), vc)
+
+
+def test_prefill_then_decode_agree(dev, orc):
+    """End to end: causal prefill over packed sequences, the same K/V written to a paged cache, and the
+    decode kernel asked for the LAST token of every sequence give the same rows."""
+    from feather_amd.routines.attention import flash_attention_fp8_varlen_acc_fp32_gpu
+    from feather_amd.routines.paged_attention import paged_attention_fp8_acc_fp32_gpu, paged_cache_write
+    rng = np.random.default_rng(9)
+    mode, n_heads, n_kv, d, bs = "E4M3", 8, 2, 64, 16
+    lens = [300, 17, 1024]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    total, max_blocks = int(cu[-1]), 64
+    q = orc.pack_fp8(rng.standard_normal((n_heads, total, d)).astype(np.float16), mode).reshape(n_heads, total, d // 4)
+    k = orc.pack_fp8(rng.standard_normal((n_kv, total, d)).astype(np.float16), mode).reshape(n_kv, total, d // 4)
+    v = orc.pack_fp8(rng.standard_normal((n_kv, total, d)).astype(np.float16), mode).reshape(n_kv, total, d // 4)
+    qd, kd, vd = (_dev_words(a, dev, a.shape) for a in (q, k, v))
+    cud = torch.from_numpy(cu).to(dev)
+    pre = flash_attention_fp8_varlen_acc_fp32_gpu(qd, kd, vd, cud, max(lens), mode=mode, causal=True)
+    n_blocks = 3 * max_blocks
+    bt = torch.from_numpy(rng.permutation(n_blocks).reshape(3, max_blocks).astype(np.int32)).to(dev)
+    kc = torch.zeros((n_blocks, n_kv, bs, d // 4), dtype=torch.int32, device=dev).view(torch.uint32)
+    vc = torch.zeros_like(kc)
+    paged_cache_write(kd, vd, kc, vc, bt, cud, mode=mode)
+    last = torch.from_numpy(cu[1:] - 1).to(dev).long()
+    q_last = qd.view(torch.int32)[:, last].permute(1, 0, 2).contiguous().view(torch.uint32)      # [n_seq, n_heads, d/4]
+    dec = paged_attention_fp8_acc_fp32_gpu(q_last, kc, vc, bt, torch.tensor(lens, dtype=torch.int32, device=dev), mode=mode)
+    want = pre[:, last].permute(1, 0, 2)
+    assert ((dec - want).abs().max() / want.abs().max()).item() <= TOL

@@ -413,3 +413,56 @@ def test_decode_ref_online_attention_matches_exact_softmax(orc):
         assert np.abs(got - want).max() / np.abs(want).max() < 1e-3
     V = np.full((50, 64), 2.5)
     assert np.allclose(decode_ref.online_attention(rng.standard_normal(50).astype(np.float32), V, 1.0), 2.5, rtol=1e-3)
+
+
+# ---------------------------------------------------------------- variable-length / causal attention, cache writer
+
+def test_attention_varlen_oracle_reduces_to_fixed_length_and_prefix(orc):
+    """Pins attention_varlen_f64_np: (a) without a mask each sequence equals the fixed-length closed
+    form on its own rows; (b) causal row i equals NON-causal attention over the prefix 0..i (the
+    definition of the mask, evaluated by the already pinned routine); (c) row 0 of a causal sequence
+    is V[0]; (d) rows outside every sequence stay zero."""
+    rng = np.random.default_rng(5)
+    d, mode, total = 64, "E5M2", 40
+    cu = [3, 12, 12, 33]                                    # a gap in front, an empty sequence, a tail gap
+    q = orc.pack_fp8(rng.standard_normal((2, total, d)).astype(np.float16), mode).reshape(2, total, d // 4)
+    k = orc.pack_fp8(rng.standard_normal((1, total, d)).astype(np.float16), mode).reshape(1, total, d // 4)
+    v = orc.pack_fp8(rng.standard_normal((1, total, d)).astype(np.float16), mode).reshape(1, total, d // 4)
+    full = orc.attention_varlen_f64_np(q, k, v, cu, d, mode)
+    caus = orc.attention_varlen_f64_np(q, k, v, cu, d, mode, causal=True)
+    for h in range(2):
+        for a, b in ((3, 12), (12, 33)):
+            want = orc.attention_f64_np(q[h, a:b].reshape(-1), k[0, a:b].reshape(-1), v[0, a:b].reshape(-1), b - a, d, mode)[0]
+            assert np.allclose(full[h, a:b], want, rtol=1e-12, atol=1e-14)
+            for i in (0, 1, (b - a) // 2, b - a - 1):
+                pre = orc.attention_f64_np(q[h, a + i:a + i + 1].repeat(i + 1, axis=0).reshape(-1), k[0, a:a + i + 1].reshape(-1),
+                                           v[0, a:a + i + 1].reshape(-1), i + 1, d, mode)[0]
+                assert np.allclose(caus[h, a + i], pre[0], rtol=1e-12, atol=1e-14)
+            assert np.allclose(caus[h, a], orc.decode_np(v[0, a], mode))
+    for o in (full, caus):
+        assert not o[:, :3].any() and not o[:, 33:].any()
+
+
+def test_paged_cache_write_oracle_places_rows(orc):
+    """Pins paged_cache_write_np by reading the cache back through the block table (gather is the
+    inverse of the scatter), untouched slots and dropped positions included."""
+    rng = np.random.default_rng(6)
+    n_kv, dw, bs, max_blocks, n_blocks = 2, 4, 4, 3, 8
+    cu = np.array([0, 5, 5, 14], dtype=np.int32)
+    start = np.array([2, 0, 6], dtype=np.int32)             # sequence 2 runs past 3 blocks x 4 slots: 3 rows dropped
+    bt = np.array([[5, 1, 7], [0, 0, 0], [2, 6, 3]], dtype=np.int32)
+    k = rng.integers(1, 2**32, (n_kv, 14, dw), dtype=np.uint64).astype(np.uint32)
+    v = rng.integers(1, 2**32, (n_kv, 14, dw), dtype=np.uint64).astype(np.uint32)
+    kc = np.zeros((n_blocks, n_kv, bs, dw), dtype=np.uint32)
+    vc = np.zeros_like(kc)
+    orc.paged_cache_write_np(k, v, kc, vc, bt, cu, start)
+    written = 0
+    for s in range(3):
+        for i in range(cu[s + 1] - cu[s]):
+            pos = start[s] + i
+            if pos >= bs * max_blocks:
+                continue
+            assert (kc[bt[s, pos // bs], :, pos % bs] == k[:, cu[s] + i]).all()
+            assert (vc[bt[s, pos // bs], :, pos % bs] == v[:, cu[s] + i]).all()
+            written += 1
+    assert written == 5 + 6 and (kc.reshape(-1, dw).any(axis=1).sum() == written * n_kv)

@@ -175,6 +175,14 @@ def main() -> int:
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_mfma_frac"] = round(flops / us / 1e6 / MFMA_PEAK_F16_TFLOPS, 4)
             us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 2, sync)
             extra[f"sdpa_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
+            if L == 8192:   # causal prefill (half the flops) vs causal fp16 SDPA
+                us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
+                                                                                    mode="E5M2", causal=True), 10, 2, sync)
+                extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
+                extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / 2 / us / 1e6, 1)
+                us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16, is_causal=True),
+                                      10, 2, sync)
+                extra[f"sdpa_causal_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
             del qkv16, pk
         torch.cuda.empty_cache()
         # paged-attention decode, 32 sequences x 32 query heads over 4 KV heads, d=64, E4M3, blocks of 16
@@ -192,7 +200,16 @@ def main() -> int:
                                                                         max_context_len=c), 50, 5, sync)
             extra[f"paged_attn_e4m3_s32_h32kv4_d64_ctx{c}_us"] = round(us, 2)
             extra[f"paged_attn_e4m3_s32_h32kv4_d64_ctx{c}_GBps"] = round(2 * n_seq * Hkv * d * c / us / 1e3, 1)
-        del kc, vc, qp
+        # prefill -> paged cache: 32 sequences x 2048 rows x 4 KV heads of packed K and V (1 B in + 1 B out per code)
+        from feather_amd.routines.paged_attention import paged_cache_write
+        rows = n_seq * 2048
+        ksrc, vsrc = (feather.pack_fp8_tensor(randn(Hkv * rows * d).half(), mode="E4M3").view(Hkv, rows, d // 4)
+                      for _ in range(2))
+        cu = torch.arange(0, rows + 1, 2048, dtype=torch.int32, device=dev)
+        us = gpu_time_us(lambda i: paged_cache_write(ksrc, vsrc, kc, vc, bt, cu, mode="E4M3"), 50, 5, sync)
+        extra["paged_cache_write_e4m3_s32_L2048_kv4_d64_us"] = round(us, 2)
+        extra["paged_cache_write_e4m3_s32_L2048_kv4_d64_GBps"] = round(4 * Hkv * rows * d / us / 1e3, 1)
+        del kc, vc, qp, ksrc, vsrc
         torch.cuda.empty_cache()
         # decode step of a TinyLlama-1.1B-shaped model (random weights), batch 32, contexts 512..4095, E4M3
         from feather_amd.routines.decode import TINYLLAMA_1_1B as cfg, PackedDecoder, random_weights

@@ -27,6 +27,9 @@ ARCH = "gfx950"
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", "-fno-gpu-rdc", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA accumulators stay in architectural VGPRs: the kernels rescale them with VALU ops, and
+    # every such touch of an AGPR accumulator costs a v_accvgpr_read/write pair
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wall", "-Wno-unused-function",
 ]
 

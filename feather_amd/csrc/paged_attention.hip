@@ -77,17 +77,50 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     __shared__ float ml_lds[kPaWaves][2][16];
     __shared__ float4_t o_lds[kPaWaves - 1][RB * 4][kWave];
 
-    // Consecutive workgroups go to consecutive XCDs.  Split-major order puts the (sequence, head)
-    // pairs of one split on all XCDs alike; with the split index fastest, all first splits (the
-    // ones every sequence has) would land on the same XCD whenever n_splits is a multiple of 8.
-    const int n_pairs = gridDim.x / n_splits;
-    const int split = blockIdx.x / n_pairs;
-    const int kvh = (blockIdx.x % n_pairs) % n_kv_heads;
-    const int seq = (blockIdx.x % n_pairs) / n_kv_heads;
-    const int group = n_q_heads / n_kv_heads;
-    const int ctx_raw = ctx_lens[seq];
-    const int t_begin = split * kSplit;
+    // Work item of this workgroup.  With one split per sequence the grid is exactly the
+    // (sequence, KV head) pairs.  Otherwise the grid is sized for max_ctx and most sequences use
+    // fewer splits: the workgroups that have work are the FIRST ones in launch order (items are
+    // numbered over the splits that exist, found from a prefix sum over the context lengths that
+    // every wave computes for itself), so the hardware spreads them over all XCDs and CUs in its
+    // first pass and the rest exit at once.  (Numbering items over the full grid left the CUs
+    // unevenly loaded; and with the split index fastest all first splits landed on one XCD,
+    // because consecutive workgroups go to consecutive XCDs.)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, kb = lane >> 4;
+    const int kvh = blockIdx.x % n_kv_heads;
+    int seq = blockIdx.x / n_kv_heads, split = 0;
+    int ctx_raw;
+    if (n_splits > 1) {
+        const int n_seq = gridDim.x / (n_splits * n_kv_heads);
+        const int item = blockIdx.x / n_kv_heads;          // index over the (sequence, split) pairs that exist
+        int base = 0;
+        seq = -1;
+        ctx_raw = 0;
+        for (int s0 = 0; s0 < n_seq && seq < 0; s0 += kWave) {
+            const int s = s0 + lane;
+            const int c = s < n_seq ? max(ctx_lens[s], 0) : 0;
+            const int ns = (min(c, max_ctx) + kSplit - 1) / kSplit;
+            int inc = ns;                                   // inclusive prefix sum over the lanes
+#pragma unroll
+            for (int off = 1; off < kWave; off <<= 1) {
+                const int t = __shfl_up(inc, off, kWave);
+                if (lane >= off) inc += t;
+            }
+            const int exc = base + inc - ns;
+            const uint64_t hit = __builtin_amdgcn_ballot_w64(item >= exc && item < exc + ns);
+            if (hit) {
+                const int src = __builtin_ctzll(hit);
+                seq = s0 + src;
+                split = item - __builtin_amdgcn_readlane(exc, src);
+                ctx_raw = __builtin_amdgcn_readlane(c, src);
+            }
+            base += __builtin_amdgcn_readlane(inc, kWave - 1);
+        }
+        if (seq < 0) return;                                // beyond the last item (whole workgroup)
+    } else {
+        ctx_raw = ctx_lens[seq];
+    }
+    const int group = n_q_heads / n_kv_heads;
+    const int t_begin = split * kSplit;
     auto blk_of = [&](int tok) { return FAST ? tok >> bs_shift : tok / block_size; };
     auto slot_of = [&](int tok) { return FAST ? tok & (block_size - 1) : tok % block_size; };
     const int32_t *bt = block_tables + (int64_t)seq * max_blocks;
@@ -162,24 +195,31 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     // Row addresses are formed right before the loads (only the block ids of the steps in flight
     // stay in registers).  Rows past the context read the fallback block (valid memory) and are
     // masked later.
-    auto row_base = [&](int blk, int tok) { return ((int64_t)blk * n_kv_heads + kvh) * block_size + slot_of(tok); };
+    // row index inside the cache in 32 bits (a cache of 2^31 rows of d codes is >= 128 GB)
+    auto row_base = [&](int blk, int tok) { return (int64_t)(uint32_t)((blk * n_kv_heads + kvh) * block_size + slot_of(tok)); };
     auto load_step = [&](Step &S, int t0) {
+        const bool full = t0 + kStepTok <= ctx;   // wave-uniform: every token of the step exists
 #pragma unroll
         for (int a = 0; a < 2; a++) {
             const int tk = t0 + 16 * a + j;
-            const uint32_t *kr = k_cache + row_base(tk < ctx ? S.kid[a] : fallback, tk) * DW;
+            const uint32_t *kr = k_cache + row_base(full || tk < ctx ? S.kid[a] : fallback, tk) * DW;
 #pragma unroll
             for (int c64 = 0; c64 < RB; c64++) S.kw[a][c64] = *reinterpret_cast<const u32x4 *>(kr + 16 * c64 + 4 * kb);
             const int tq = t0 + 16 * a + 4 * kb;
             const uint32_t *vq = nullptr;
             if constexpr (FAST)                   // an aligned group of 4 tokens shares a block
-                vq = v_cache + row_base(tq < ctx ? S.vid[a][0] : fallback, tq) * DW + j;
+                vq = v_cache + row_base(full || tq < ctx ? S.vid[a][0] : fallback, tq) * DW + j;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const uint32_t *vr = vq + r * DW;
-                if constexpr (!FAST) vr = v_cache + row_base(tq + r < ctx ? S.vid[a][r] : fallback, tq + r) * DW + j;
+                if constexpr (!FAST) vr = v_cache + row_base(full || tq + r < ctx ? S.vid[a][r] : fallback, tq + r) * DW + j;
+                if (full) {
 #pragma unroll
-                for (int rb = 0; rb < RB; rb++) S.vw[rb][a][r] = tq + r < ctx ? vr[16 * rb] : 0u;
+                    for (int rb = 0; rb < RB; rb++) S.vw[rb][a][r] = vr[16 * rb];
+                } else {
+#pragma unroll
+                    for (int rb = 0; rb < RB; rb++) S.vw[rb][a][r] = tq + r < ctx ? vr[16 * rb] : 0u;
+                }
             }
         }
     };
@@ -194,32 +234,41 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
                 s[a] = pa_mfma16(pa_dec8<MODE>(S.kw[a][c64].z, S.kw[a][c64].w), qf[2 * c64 + 1], s[a]);
             }
         }
-        // online softmax (lane column = query head), log2 domain
-        float mx = -INFINITY;
+        // online softmax (lane column = query head), log2 domain; only the last step of a split
+        // can hold tokens past its end (wave-uniform test)
+        if (t0 + kStepTok > t_end) {
 #pragma unroll
-        for (int a = 0; a < 2; a++)
+            for (int a = 0; a < 2; a++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                float x = s[a][r] * scale_log2e;
-                if (t0 + 16 * a + 4 * kb + r >= t_end) x = -INFINITY;
-                s[a][r] = x;
-                mx = fmaxf(mx, x);
-            }
+                for (int r = 0; r < 4; r++)
+                    if (t0 + 16 * a + 4 * kb + r >= t_end) s[a][r] = -INFINITY;
+        }
+        float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                         fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
         mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
         mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-        float m_new = fmaxf(m_run, mx);
-        float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
+        const float m_new = fmaxf(m_run, mx * scale_log2e);      // scale > 0: the maximum commutes with it
         half8_t p8;
         float rs = 0.f;
 #pragma unroll
         for (int a = 0; a < 2; a++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                float e = __builtin_amdgcn_exp2f(s[a][r] - m_new);
+                float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[a][r], scale_log2e, -m_new));
                 rs += e;
                 p8[4 * a + r] = (_Float16)e;
             }
+        // rescale only when some query head of the wave saw a new maximum (wave-uniform test)
+        const bool moved = __builtin_amdgcn_ballot_w64(m_new != m_run) != 0;
+        float alpha = 1.0f;
+        if (moved) {
+            alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) o[rb][c] *= alpha;
+        }
         l_run = l_run * alpha + rs;
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
@@ -231,7 +280,7 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 u32x4 vf = u32x4{pr[0][c], pr[1][c], pr[2][c], pr[3][c]};
-                o[rb][c] = pa_mfma16(__builtin_bit_cast(half8_t, vf), p8, o[rb][c] * alpha);
+                o[rb][c] = pa_mfma16(__builtin_bit_cast(half8_t, vf), p8, o[rb][c]);
             }
         }
     };
@@ -447,6 +496,7 @@ extern "C" int feather_paged_attn_fp8(const void *q, const void *k_cache, const 
     FEATHER_CHECK(d == 64 || d == 128 || d == 256, FEATHER_ESHAPE, "%s: head dim %lld not supported (64, 128, 256)", me,
                   (long long)d);
     FEATHER_CHECK(max_ctx <= max_blocks * block_size, FEATHER_ESHAPE, "%s: max_ctx exceeds the block table", me);
+    FEATHER_CHECK(scale > 0.f, FEATHER_EINVAL, "%s: scale must be positive (the running maximum is kept on raw scores)", me);
     if (n_seq == 0) return FEATHER_OK;
     FEATHER_CHECK(q && k_cache && v_cache && block_tables && ctx_lens && out_f32 && scratch, FEATHER_EINVAL,
                   "%s: null pointer", me);

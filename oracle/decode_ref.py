@@ -72,7 +72,9 @@ def online_attention(dots: np.ndarray, V: np.ndarray, scale: float, chunk: int =
                 xs = x[c0:min(c0 + chunk, s1)]
                 m_new = max(m, float(xs.max()))
                 alpha = np.float32(np.exp2(np.float32(m - m_new))) if np.isfinite(m) else np.float32(0)
-                p = np.exp2((xs - np.float32(m_new)).astype(np.float32)).astype(np.float32)
+                # the kernel evaluates 2^(s * c - m) with one fused multiply-add per score
+                raw = dots[c0:min(c0 + chunk, s1)].astype(np.float32).astype(np.float64)
+                p = np.exp2((raw * float(c) - m_new).astype(np.float32)).astype(np.float32)
                 l = np.float32(l * alpha + p.sum(dtype=np.float32))
                 o = o * float(alpha) + p.astype(np.float16).astype(np.float64) @ V[c0:c0 + len(xs)]
                 m = m_new

@@ -78,20 +78,20 @@ __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t 
 #pragma unroll
         for (int i = 0; i < NB; i++) xr[i] = xok[i] ? *reinterpret_cast<const u32x4 *>(xp[i] + col) : u32x4{0, 0, 0, 0};
     };
-    if (c_begin < c_end) issue(c_begin, wa, xa);
-    for (int c = c_begin; c < c_end; c++) {
+    // One chunk: vectors' chunk -> LDS, (the caller's prefetch goes here), barrier, MFMAs.
+    auto stage_x = [&](int c, const u32x4 (&xr)[NB]) {
         _Float16 *buf = xs + ((c - c_begin) & 1) * (16 * NB * kBgPitch);
 #pragma unroll
         for (int i = 0; i < NB; i++) {
-            *reinterpret_cast<half8_t *>(buf + xdst[i]) = bg_dec8<MODE>(xa[i].x, xa[i].y);
-            *reinterpret_cast<half8_t *>(buf + xdst[i] + 8) = bg_dec8<MODE>(xa[i].z, xa[i].w);
+            *reinterpret_cast<half8_t *>(buf + xdst[i]) = bg_dec8<MODE>(xr[i].x, xr[i].y);
+            *reinterpret_cast<half8_t *>(buf + xdst[i] + 8) = bg_dec8<MODE>(xr[i].z, xr[i].w);
         }
-        u32x4 wn[4], xn[NB];
-        if (c + 1 < c_end) issue(c + 1, wn, xn);
-        __syncthreads();
+        return buf;
+    };
+    auto mac = [&](const _Float16 *buf, const u32x4 (&wr)[4]) {
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            half8_t a0 = bg_dec8<MODE>(wa[u].x, wa[u].y), a1 = bg_dec8<MODE>(wa[u].z, wa[u].w);
+            half8_t a0 = bg_dec8<MODE>(wr[u].x, wr[u].y), a1 = bg_dec8<MODE>(wr[u].z, wr[u].w);
 #pragma unroll
             for (int nb = 0; nb < NB; nb++) {
                 const _Float16 *b = buf + (16 * nb + j) * kBgPitch + 64 * u + 16 * kb;
@@ -99,12 +99,27 @@ __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t 
                 acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, *reinterpret_cast<const half8_t *>(b + 8), acc[nb], 0, 0, 0);
             }
         }
-        if (c + 1 < c_end) {
+    };
+    if (c_begin >= c_end) return;                  // cannot happen: the launcher creates no empty slice
+    issue(c_begin, wa, xa);
+    // Every chunk but the last prefetches its successor unconditionally, so the number of loads
+    // in flight is known at compile time and the wait for chunk c leaves chunk c + 1 outstanding
+    // (a prefetch inside an `if` makes the compiler wait for everything).
+    for (int c = c_begin; c < c_end - 1; c++) {
+        const _Float16 *buf = stage_x(c, xa);
+        u32x4 wn[4], xn[NB];
+        issue(c + 1, wn, xn);
+        __syncthreads();
+        mac(buf, wa);
 #pragma unroll
-            for (int u = 0; u < 4; u++) wa[u] = wn[u];
+        for (int u = 0; u < 4; u++) wa[u] = wn[u];
 #pragma unroll
-            for (int i = 0; i < NB; i++) xa[i] = xn[i];
-        }
+        for (int i = 0; i < NB; i++) xa[i] = xn[i];
+    }
+    {
+        const _Float16 *buf = stage_x(c_end - 1, xa);
+        __syncthreads();
+        mac(buf, wa);
     }
     float *o_base = out + (int64_t)blockIdx.y * part_stride;
     const int r = row0 + 4 * kb;                   // accumulator rows 4 kb + {0..3}, column = vector

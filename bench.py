@@ -211,25 +211,30 @@ def main() -> int:
         extra["paged_cache_write_e4m3_s32_L2048_kv4_d64_GBps"] = round(4 * Hkv * rows * d / us / 1e3, 1)
         del kc, vc, qp, ksrc, vsrc
         torch.cuda.empty_cache()
-        # decode step of a TinyLlama-1.1B-shaped model (random weights), batch 32, contexts 512..4095, E4M3
+        # decode step of a TinyLlama-1.1B-shaped model (random weights), contexts 512..4095: batch 32 in E4M3
+        # (the configuration of the metric), then E5M2 and batch 64 for comparison
         from feather_amd.routines.decode import TINYLLAMA_1_1B as cfg, PackedDecoder, random_weights
-        wts = random_weights(cfg, seed=5, device=dev)
-        dec = PackedDecoder(cfg, wts, n_blocks=nblk, max_blocks=cmax // bs, mode="E4M3", device=dev)
-        del wts
-        for lay in dec.layers:
-            for name in ("k_cache", "v_cache"):
-                vals = randn(nblk * cfg.n_kv_heads * bs * cfg.head_dim).half()
-                lay[name].view(-1).copy_(feather.pack_fp8_tensor(vals, mode="E4M3").view(torch.int32))
-        cl = torch.randint(512, cmax, (n_seq,), generator=g, device=dev, dtype=torch.int32)
-        tok = torch.randint(0, cfg.vocab, (n_seq,), generator=g, device=dev, dtype=torch.int32)
-        logits = torch.empty((n_seq, cfg.vocab), dtype=torch.float32, device=dev)
-        us = gpu_time_us(lambda i: dec.step(tok, bt, cl, out=logits), 20, 3, sync)
-        step_bytes = dec.weight_bytes() + int(cl.sum().item()) * 2 * cfg.n_kv_heads * cfg.head_dim * cfg.n_layers
-        extra["decode_tinyllama_b32_e4m3_ms_per_step"] = round(us / 1e3, 3)
-        extra["decode_tinyllama_b32_e4m3_tokens_per_s"] = round(n_seq / us * 1e6, 0)
-        extra["decode_tinyllama_b32_e4m3_GBps"] = round(step_bytes / us / 1e3, 1)
-        del dec, logits
-        torch.cuda.empty_cache()
+        for batch, mode in ((32, "E4M3"), (32, "E5M2"), (64, "E4M3")):
+            nb_ = batch * cmax // bs
+            wts = random_weights(cfg, seed=5, device=dev)
+            dec = PackedDecoder(cfg, wts, n_blocks=nb_, max_blocks=cmax // bs, mode=mode, device=dev)
+            del wts
+            for lay in dec.layers:
+                for name in ("k_cache", "v_cache"):
+                    vals = randn(nb_ * cfg.n_kv_heads * bs * cfg.head_dim).half()
+                    lay[name].view(-1).copy_(feather.pack_fp8_tensor(vals, mode=mode).view(torch.int32))
+            btd = torch.randperm(nb_, generator=g, device=dev).to(torch.int32).view(batch, cmax // bs)
+            cl = torch.randint(512, cmax, (batch,), generator=g, device=dev, dtype=torch.int32)
+            tok = torch.randint(0, cfg.vocab, (batch,), generator=g, device=dev, dtype=torch.int32)
+            logits = torch.empty((batch, cfg.vocab), dtype=torch.float32, device=dev)
+            us = gpu_time_us(lambda i: dec.step(tok, btd, cl, out=logits), 20, 3, sync)
+            step_bytes = dec.weight_bytes() + int(cl.sum().item()) * 2 * cfg.n_kv_heads * cfg.head_dim * cfg.n_layers
+            key = f"decode_tinyllama_b{batch}_{mode.lower()}"
+            extra[key + "_ms_per_step"] = round(us / 1e3, 3)
+            extra[key + "_tokens_per_s"] = round(batch / us * 1e6, 0)
+            extra[key + "_GBps"] = round(step_bytes / us / 1e3, 1)
+            del dec, logits, btd
+            torch.cuda.empty_cache()
 
     cpu = None
     if not args.no_cpu:

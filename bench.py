@@ -159,7 +159,17 @@ def main() -> int:
         for mode in ("E5M2", "E4M3"):
             us = gpu_time_us(lambda i: feather.pack_fp8_tensor(src, mode=mode), 20, 3, sync)
             extra[f"pack_{mode.lower()}_134M_GBps"] = round(3 * src.numel() / us / 1e3, 1)
-        del src
+        # unpack (1 B in, 4 B fp32 out per element), ReLU on packed E5M2, fp16 container (2 B in + 2 B out)
+        from feather_amd.routines.activations import relu1d_fp8_ret_fp32_feather_gpu
+        words = mats["E5M2"][0][: src.numel() // 4]
+        for mode, sem in (("E4M3", "ieee"), ("E4M3", "kernel"), ("E5M2", "ieee")):
+            us = gpu_time_us(lambda i: feather.unpack_fp8_tensor(words, mode=mode, semantics=sem), 20, 3, sync)
+            extra[f"unpack_{mode.lower()}_{sem}_f32_134M_GBps"] = round(5 * src.numel() / us / 1e3, 1)
+        us = gpu_time_us(lambda i: relu1d_fp8_ret_fp32_feather_gpu(words, src.numel()), 20, 3, sync)
+        extra["relu_e5m2_f32_134M_GBps"] = round(5 * src.numel() / us / 1e3, 1)
+        us = gpu_time_us(lambda i: feather.pack_fp16_tensor(src), 20, 3, sync)
+        extra["pack_fp16_134M_GBps"] = round(4 * src.numel() / us / 1e3, 1)
+        del src, words
         del mats["E5M2"], sub, xs
         torch.cuda.empty_cache()
         # flash attention, B4 H16 d64, E5M2, vs fp16 SDPA on the same GPU

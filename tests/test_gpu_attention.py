@@ -147,6 +147,41 @@ def test_paged_attention_vs_oracle(dev, orc, mode, n_seq, Hq, Hkv, d, bs, max_ct
     assert _nerr(out.cpu().numpy(), want) <= TOL
 
 
+@pytest.mark.parametrize("mode,n_seq,Hq,Hkv,d,bs,max_ctx", [
+    ("E4M3", 70, 4, 2, 64, 16, 1100),      # more sequences than lanes of a wave, three splits
+    ("E5M2", 5, 8, 2, 64, 12, 700),        # block size that is not a power of two, two splits
+    ("E4M3", 3, 6, 3, 128, 4, 1030),       # smallest power-of-two block, three splits, d = 128
+])
+def test_paged_attention_split_bookkeeping(dev, orc, mode, n_seq, Hq, Hkv, d, bs, max_ctx):
+    """Contexts of every kind under one context bound: empty, one token, exactly one split, one token
+    more, the bound itself.  Empty sequences give zero rows."""
+    from feather_amd.routines.paged_attention import paged_attention_fp8_acc_fp32_gpu
+    rng = np.random.default_rng(n_seq + bs + max_ctx)
+    max_blocks = (max_ctx + bs - 1) // bs
+    n_blocks = n_seq * max_blocks + 1
+    ctx = rng.integers(0, max_ctx + 1, size=n_seq).astype(np.int32)
+    ctx[: 5] = [0, 1, 512, 513, max_ctx][: min(5, n_seq)]
+    if n_seq > 5:
+        ctx[-1] = 0
+    kc = orc.pack_fp8(rng.standard_normal((n_blocks, Hkv, bs, d)).astype(np.float16), mode).reshape(n_blocks, -1)
+    vc = orc.pack_fp8(rng.standard_normal((n_blocks, Hkv, bs, d)).astype(np.float16), mode).reshape(n_blocks, -1)
+    poison = n_blocks - 1                                      # a block of NaN codes: using it shows in the result
+    kc[poison] = vc[poison] = 0x7F7F7F7F
+    q = orc.pack_fp8(rng.standard_normal((n_seq, Hq, d)).astype(np.float16), mode)
+    bt = rng.permutation(n_blocks - 1)[: n_seq * max_blocks].reshape(n_seq, max_blocks).astype(np.int32)
+    for i in range(n_seq):                                     # entries past a context must never be used
+        bt[i, (ctx[i] + bs - 1) // bs:] = poison
+    out = paged_attention_fp8_acc_fp32_gpu(
+        _dev_words(q, dev, (n_seq, Hq, d // 4)), _dev_words(kc, dev, (n_blocks, Hkv, bs, d // 4)),
+        _dev_words(vc, dev, (n_blocks, Hkv, bs, d // 4)), torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev),
+        mode=mode, max_context_len=max_ctx).cpu().numpy()
+    live = np.flatnonzero(ctx > 0)
+    want = orc.paged_attn(q.reshape(n_seq, -1)[live], kc, vc, bt[live], ctx[live], Hq, Hkv, d, bs, mode)
+    assert np.isfinite(want).all()
+    assert _nerr(out[live], want) <= TOL
+    assert not out[ctx == 0].any()
+
+
 def test_paged_attention_config_shape(dev, orc):
     """TinyLlama-shaped decode attention: batch 32, 32 query / 4 KV heads, d 64, block 16,
     contexts uniform in [512, 4096], permuted block table."""

@@ -260,7 +260,7 @@ def main() -> int:
         "value": round(kern_us, 3), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "E4M3 packed GEMV 16384x16384 + vector 16384 (BASELINE configs[1]); N(0,1) fp16 "
+        "config": {"workload": "E4M3 packed GEMV 16384x16384 + vector 16384 (the configuration the metric is quoted on); N(0,1) fp16 "
                                "sources with 1% of entries x1e-3, packed 4 codes per 32-bit word; 4 distinct "
                                "matrices (1 GiB) rotated",
                    "M": M, "K": K, "mode": "E4M3", "buffers": NBUF},

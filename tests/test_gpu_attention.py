@@ -121,6 +121,31 @@ def test_flash_attention_config_sized_property(dev):
     assert torch.equal(out, again)
 
 
+@pytest.mark.parametrize("mode,B,H,L,d,causal", [
+    ("E5M2", 4, 16, 8192, 64, False), ("E4M3", 1, 8, 4096, 256, False), ("E4M3", 1, 8, 8192, 512, False),
+    ("E4M3", 1, 8, 1024, 256, True), ("E5M2", 2, 4, 8192, 64, True),
+])
+def test_flash_attention_full_size_rows_vs_fp32_math(dev, mode, B, H, L, d, causal):
+    """The remaining attention shapes of the benchmark configurations, too big for the scalar oracle:
+    a sample of query rows of two heads against explicit fp32 softmax(q K^T / sqrt(d)) V of the
+    decoded operands (float64 accumulation on the device)."""
+    import feather_amd as feather
+    g = torch.Generator(device=dev).manual_seed(L + d)
+    qkv = [torch.randn(B, H, L, d, generator=g, device=dev).half() for _ in range(3)]
+    p = [feather.pack_fp8_tensor(t, mode=mode).view(B, H, L, d // 4) for t in qkv]
+    out = feather.flash_attention_fp8_acc_fp32_gpu(p[0], p[1], p[2], L, d // 4, mode=mode, causal=causal)
+    assert out.shape == (B, H, L, d) and bool(torch.isfinite(out).all())
+    dec = [feather.unpack_fp8_tensor(t, mode=mode, semantics="kernel", dtype=torch.float32).view(B, H, L, d).double() for t in p]
+    rows = torch.tensor([0, 1, 63, 64, L // 2 - 1, L // 2, L - 2, L - 1], device=dev)
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        s = dec[0][b, h, rows] @ dec[1][b, h].T / (d ** 0.5)               # [rows, L]
+        if causal:
+            s = s.masked_fill(torch.arange(L, device=dev)[None, :] > rows[:, None], float("-inf"))
+        want = torch.softmax(s, dim=-1) @ dec[2][b, h]
+        err = (out[b, h, rows].double() - want).abs().max() / want.abs().max()
+        assert err.item() <= TOL
+
+
 # ---------------------------------------------------------------- paged decode
 
 @pytest.mark.parametrize("mode,n_seq,Hq,Hkv,d,bs,max_ctx", [

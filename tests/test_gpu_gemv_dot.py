@@ -154,6 +154,24 @@ def test_gemv_batched_vs_oracle(dev, orc, mode, M, K, nvec):
         assert _nerr(out, orc.gemv_batched(wp, xp, M, K, nvec, mode)) <= TOL
 
 
+@pytest.mark.parametrize("M,K", [(32000, 2048), (11264, 2048), (2048, 5632), (2560, 2048)])
+def test_gemv_batched_decode_shapes_vs_fp64_math(dev, M, K):
+    """The weight shapes of the TinyLlama-shaped decode step at batch 32, E4M3: against a float64
+    matmul of the decoded operands on the device (the scalar oracle is too slow here)."""
+    import feather_amd as feather
+    from feather_amd.routines.gemv import gemv_fp8_batched_acc_fp32_gpu
+    g = torch.Generator(device=dev).manual_seed(M + K)
+    w16 = (torch.randn(M, K, generator=g, device=dev) / K ** 0.5).half()
+    x16 = torch.randn(32, K, generator=g, device=dev).half()
+    wp, xp = feather.pack_fp8_tensor(w16, mode="E4M3"), feather.pack_fp8_tensor(x16, mode="E4M3")
+    out = gemv_fp8_batched_acc_fp32_gpu(wp, xp, (M, K), 32, "E4M3")
+    wd = feather.unpack_fp8_tensor(wp, mode="E4M3", semantics="kernel").view(M, K).double()
+    xd = feather.unpack_fp8_tensor(xp, mode="E4M3", semantics="kernel").view(32, K).double()
+    want = xd @ wd.T
+    assert out.shape == (32, M)
+    assert ((out.double() - want).abs().max() / want.abs().max()).item() <= TOL
+
+
 # ---------------------------------------------------------------- dot
 
 def test_dot_docstring_known_answers(dev, kats):

@@ -54,6 +54,38 @@ def test_decode_step_vs_oracle(orc, mode, hidden, nq, nkv, inter):
         ctx = ctx + 1
 
 
+def test_decode_step_long_contexts_use_split_attention(orc):
+    """Contexts longer than one 512-token split: the attention of the step runs as several splits
+    plus the merge kernel that emits the packed operand of W_o."""
+    import feather_amd as feather
+    from feather_amd.routines.decode import DecoderConfig, PackedDecoder, random_weights
+    from oracle import decode_ref
+    dev = torch.device("cuda:0")
+    mode = "E4M3"
+    cfg = DecoderConfig(n_layers=1, hidden=256, n_q_heads=4, n_kv_heads=2, head_dim=64, inter=512, vocab=300)
+    B, max_blocks = 4, 80                                     # up to 1280 tokens: three splits
+    n_blocks = B * max_blocks
+    w = random_weights(cfg, seed=3)
+    dec = PackedDecoder(cfg, w, n_blocks=n_blocks, max_blocks=max_blocks, mode=mode, device=dev)
+    g = torch.Generator().manual_seed(2)
+    bt = torch.randperm(n_blocks, generator=g).to(torch.int32).view(B, max_blocks)
+    ctx = torch.tensor([700, 1279, 512, 3], dtype=torch.int32)
+    dw = cfg.head_dim // 4
+    vals = [torch.randn(n_blocks, cfg.n_kv_heads, cfg.block_size, cfg.head_dim, generator=g).half() for _ in range(2)]
+    packed = [feather.pack_fp8_tensor(v.to(dev), mode=mode).view(n_blocks, cfg.n_kv_heads, cfg.block_size, dw) for v in vals]
+    dec.layers[0]["k_cache"].copy_(packed[0].view(torch.int32))
+    dec.layers[0]["v_cache"].copy_(packed[1].view(torch.int32))
+    kc_np = [packed[0].view(torch.int32).cpu().numpy().view(np.uint32).copy()]
+    vc_np = [packed[1].view(torch.int32).cpu().numpy().view(np.uint32).copy()]
+    tokens = torch.randint(0, cfg.vocab, (B,), generator=g, dtype=torch.int32)
+    logits = dec.step(tokens.to(dev), bt.to(dev), ctx.to(dev)).cpu().numpy()
+    want = decode_ref.decode_step_ref(cfg, {k: v.numpy() for k, v in w.items()}, kc_np, vc_np, tokens.numpy(), bt.numpy(),
+                                      ctx.numpy(), mode)
+    assert np.abs(logits - want).max() / np.abs(want).max() <= 2e-2
+    got_k = dec.layers[0]["k_cache"].cpu().numpy().view(np.uint32)
+    assert np.mean(got_k.view(np.uint8) == kc_np[0].view(np.uint8)) >= 0.9999
+
+
 def test_decode_step_rejects_bad_arguments():
     from feather_amd.routines.decode import DecoderConfig, PackedDecoder, random_weights
     dev = torch.device("cuda:0")

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t 
     auto issue = [&](int c, u32x4 (&wr)[4], u32x4 (&xr)[NB]) {
         const int64_t col = (int64_t)c * kBgChunk;
 #pragma unroll
-        for (int u = 0; u < 4; u++) wr[u] = load_nt128(wp + col + 64 * u);
+        for (int u = 0; u < 4; u++) wr[u] = *reinterpret_cast<const u32x4 *>(wp + col + 64 * u);
 #pragma unroll
         for (int i = 0; i < NB; i++) xr[i] = xok[i] ? *reinterpret_cast<const u32x4 *>(xp[i] + col) : u32x4{0, 0, 0, 0};
     };

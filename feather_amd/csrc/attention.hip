@@ -111,7 +111,7 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
         keys_scored = (last_key + BN - 1) / BN * BN;
     }
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = wave_id();
     const int j = lane & 15, kb = lane >> 4;
     const int q0 = tile * QT + wave * (16 * QB);
 

@@ -202,4 +202,9 @@ __device__ __forceinline__ float wave_sum(float x) {
 
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }
 
+// Index of the wave inside its workgroup, marked as wave-uniform: everything derived from it (row
+// bases, query offsets, step indices) then lives in SGPRs and is computed on the scalar unit
+// instead of once per lane (the compiler cannot see that threadIdx.x / 64 is uniform).
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave)); }
+
 }  // namespace feather

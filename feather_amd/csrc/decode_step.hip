@@ -23,7 +23,7 @@ constexpr int kDsThreads = 256;
 
 __device__ __forceinline__ float block_sum(float x, float *red) {
     x = wave_sum(x);
-    const int lane = lane_id(), wave = threadIdx.x / kWave;
+    const int lane = lane_id(), wave = wave_id();
     if (lane == 0) red[wave] = x;
     __syncthreads();
     float t = 0.f;

@@ -86,7 +86,7 @@ __global__ __launch_bounds__(kDotThreads) void dot_kernel(const uint32_t *__rest
     for (int64_t j = done + tid; j < n_words; j += nthreads) acc[0] = mac_word<KIND>(x1[j], x2[j], acc[0]);
 
     float s = wave_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
-    const int lane = lane_id(), wave = threadIdx.x / kWave;
+    const int lane = lane_id(), wave = wave_id();
     if (lane == 0) wave_part[wave] = s;
     __syncthreads();
     if (threadIdx.x == 0) {

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(WAVES * kWave) void gemv_fp8_kernel(const uint8_t *
     __syncthreads();
 
     const int lane = lane_id();
-    const int wave = threadIdx.x / kWave;
+    const int wave = wave_id();
     const int row_begin = blockIdx.x * rows_per_wg;
     const int row_end = min(row_begin + rows_per_wg, M);
     const u32x4 *lds128 = reinterpret_cast<const u32x4 *>(lds32);
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_fp8_generic_kernel(const ui
                                                                        const uint32_t *__restrict__ v,
                                                                        float *__restrict__ out, int M, int64_t n_col) {
     const int lane = lane_id();
-    const int wave = threadIdx.x / kWave;
+    const int wave = wave_id();
     for (int row = blockIdx.x * kGemvWaves + wave; row < M; row += gridDim.x * kGemvWaves) {
         const uint32_t *rp = m + (int64_t)row * n_col;
         float acc = 0.f;

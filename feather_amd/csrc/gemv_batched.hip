@@ -47,7 +47,7 @@ __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t 
                                                                  float *__restrict__ out, int M, int K, int nvec,
                                                                  int cps, int64_t part_stride) {
     extern __shared__ __attribute__((aligned(16))) _Float16 xs[];   // [2][16 * NB][kBgPitch]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_id();
     const int j = lane & 15, kb = lane >> 4;
     const int row0 = blockIdx.x * kBgRows + 16 * wave;
     const int row = min(row0 + j, M - 1);

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     // first pass and the rest exit at once.  (Numbering items over the full grid left the CUs
     // unevenly loaded; and with the split index fastest all first splits landed on one XCD,
     // because consecutive workgroups go to consecutive XCDs.)
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, kb = lane >> 4;
+    const int lane = threadIdx.x & 63, wave = wave_id(), j = lane & 15, kb = lane >> 4;
     const int kvh = blockIdx.x % n_kv_heads;
     int seq = blockIdx.x / n_kv_heads, split = 0;
     int ctx_raw;

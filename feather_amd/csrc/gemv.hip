@@ -14,13 +14,18 @@
 //     added into an fp32 accumulator);
 //   * the RPW row sums are folded across the wave with DPP.
 //
-// Two measured dead ends, kept here so they are not tried again.  (1) Feeding
+// Measured dead ends, kept here so they are not tried again.  (1) Feeding
 // the codes to FP8 MFMAs (matrix bytes as A, vector bytes as B, dot product on
 // the diagonal of the 16x16 result) removes the decode but ran 12 % SLOWER at
 // 16384^2 (47.3 us against 41.6 us for E5M2).  (2) Issuing the loads of the
 // next group before the arithmetic of the current one (software pipelining,
 // twice the bytes in flight) also lost 6 %: at ~6.4 TB/s the memory system is
-// saturated and deeper queues only add latency.
+// saturated and deeper queues only add latency.  (3) The multiply-accumulate on
+// v_mfma_f32_4x4x4f16 (one MFMA issue per packed word instead of two v_dot2c;
+// the lane's dot product sits on the diagonal of its 4x4 block) is exact and
+// changes nothing: E4M3 45.2 us either way.  (4) Plain instead of non-temporal
+// loads: 48.8 us.  Buffer loads (any cache policy) instead of global loads: no
+// gain once the row bases are wave-uniform.
 //
 // A workgroup takes a contiguous range of rows so the vector decode is
 // amortised; ranges are sized so that the grid is a few workgroups per CU.

@@ -88,8 +88,7 @@ class PackedDecoder:
                             cfg.block_size, self.max_blocks, self.code, cfg.rms_eps, cfg.rope_theta,
                             ctypes.cast(self._c_layers, ctypes.POINTER(N.DecoderLayer)), self.embed.data_ptr(),
                             self.norm_final.data_ptr(), self.lm_head.data_ptr())
-        self._scratch = None
-        self._scratch_key = None
+        self._scratch = {}
 
     def weight_bytes(self) -> int:
         """Packed weight bytes one step streams (each linear layer once, embedding rows aside)."""
@@ -114,14 +113,16 @@ class PackedDecoder:
         if block_tables.shape != (batch, self.max_blocks) or ctx_lens.shape != (batch,):
             raise ValueError("block_tables must be [batch, max_blocks] and ctx_lens [batch]")
         max_ctx = self.max_blocks * cfg.block_size if max_ctx is None else int(max_ctx)
+        # one scratch buffer per (shape, stream): steps on different streams may run concurrently
         key = (batch, max_ctx, N.stream_ptr(self.device))
-        if self._scratch_key != key:
+        if key not in self._scratch:
             nbytes = int(N.lib().feather_decode_step_scratch_bytes(ctypes.byref(self._c), batch, max_ctx))
             if nbytes < 0:
                 raise ValueError(N.lib().feather_last_error().decode())
-            self._scratch = torch.empty(nbytes + 256, dtype=torch.uint8, device=self.device)
-            self._scratch_key = key
-        sptr = (self._scratch.data_ptr() + 255) // 256 * 256
+            if len(self._scratch) >= 8:
+                self._scratch.clear()
+            self._scratch[key] = torch.empty(nbytes + 256, dtype=torch.uint8, device=self.device)
+        sptr = (self._scratch[key].data_ptr() + 255) // 256 * 256
         if out is None:
             out = torch.empty((batch, cfg.vocab), dtype=torch.float32, device=self.device)
         N.call(self.device, "feather_decode_step", ctypes.addressof(self._c), N.ptr(token_ids), N.ptr(block_tables),

@@ -60,7 +60,7 @@ def flash_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: torch.
     if causal:
         if tail != "mask":
             raise ValueError("causal attention needs tail='mask'")
-        cu = torch.tensor([0, seq_len], dtype=torch.int32, device=q.device)
+        cu = torch.arange(2, dtype=torch.int32, device=q.device) * seq_len   # [0, L], built on the device (graph-capturable)
         N.call(q.device, "feather_flash_attn_fp8_varlen", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(cu), 1, seq_len, seq_len, n_heads, d, kv_group, code, float(scale), 1)
     else:
         N.call(q.device, "feather_flash_attn_fp8", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), n_heads, seq_len, d, kv_group, code, float(scale), _TAILS[tail])

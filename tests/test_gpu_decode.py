@@ -103,3 +103,64 @@ def test_decode_step_rejects_bad_arguments():
         dec.step(tok, bt, ctx, max_ctx=1000)
     with pytest.raises(NotImplementedError):
         PackedDecoder(cfg, random_weights(cfg), n_blocks=8, max_blocks=4, mode="E3M4", device=dev)
+
+
+def test_entry_points_replay_in_a_graph():
+    """Every entry point only enqueues kernels on the caller's stream (no allocation, memset or
+    synchronisation), so a captured sequence of calls replays to the same bits as the eager run:
+    GEMV, dot, flash attention, paged attention and a decode step, replayed three times with other
+    work in between."""
+    import feather_amd as feather
+    from feather_amd.routines.decode import DecoderConfig, PackedDecoder, random_weights
+    from feather_amd.routines.paged_attention import paged_attention_fp8_acc_fp32_gpu
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(4)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev)
+    M, K = 512, 1024
+    mp, vp = feather.pack_fp8_tensor(rn(M, K).half(), mode="E4M3"), feather.pack_fp8_tensor(rn(K).half(), mode="E4M3")
+    qkv = [feather.pack_fp8_tensor(rn(2, 256, 64).half(), mode="E5M2").view(2, 256, 16) for _ in range(3)]
+    cfg = DecoderConfig(n_layers=2, hidden=256, n_q_heads=4, n_kv_heads=2, head_dim=64, inter=512, vocab=200)
+    B, max_blocks = 3, 48                                      # contexts up to 768: two attention splits
+    dec = PackedDecoder(cfg, random_weights(cfg, seed=1), n_blocks=B * max_blocks, max_blocks=max_blocks, mode="E4M3", device=dev)
+    for lay in dec.layers:
+        for name in ("k_cache", "v_cache"):
+            lay[name].view(-1).copy_(feather.pack_fp8_tensor(rn(lay[name].numel() * 4).half(), mode="E4M3").view(torch.int32))
+    bt = torch.randperm(B * max_blocks, generator=g, device=dev).to(torch.int32).view(B, max_blocks)
+    ctx = torch.tensor([700, 30, 513], dtype=torch.int32, device=dev)
+    tok = torch.tensor([1, 2, 3], dtype=torch.int32, device=dev)
+    q1 = feather.pack_fp8_tensor(rn(B, 4, 64).half(), mode="E4M3").view(B, 4, 16)
+
+    def work():
+        y = feather.gemv(mp, vp, original_shape=(M, K), mode="E4M3")
+        d = feather.dot(mp, mp, mode="E4M3")
+        a = feather.flash_attention_fp8_acc_fp32_gpu(qkv[0], qkv[1], qkv[2], 256, 16, mode="E5M2", causal=True)
+        p = paged_attention_fp8_acc_fp32_gpu(q1, dec.layers[0]["k_cache"], dec.layers[0]["v_cache"], bt, ctx, mode="E4M3")
+        lg = dec.step(tok, bt, ctx)
+        return y, d, a, p, lg
+
+    caches0 = [(lay["k_cache"].clone(), lay["v_cache"].clone()) for lay in dec.layers]
+    def reset():
+        for lay, (k0, v0) in zip(dec.layers, caches0):
+            lay["k_cache"].copy_(k0); lay["v_cache"].copy_(v0)
+
+    eager = [t.clone() for t in work()]
+    reset()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()                                                 # warm-up on a side stream (allocations happen here)
+    torch.cuda.current_stream().wait_stream(side)
+    reset()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = work()
+    for _ in range(3):
+        reset()
+        for t in outs:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(outs, eager):
+            assert torch.equal(got, want)
+        feather.gemv(mp, vp, original_shape=(M, K), mode="E4M3")   # eager work between the replays

@@ -5,6 +5,13 @@ algorithms, built by ``oracle/Makefile``) and adds numpy helpers that reduce the
 same semantics to textbook routines (LUT decode followed by a float64 matmul or
 an explicit softmax).  Only tests, the smoke check and the bench's CPU-baseline
 leg may import this package; the product package never does.
+
+Parity status of the numpy helpers defined here (the C functions list theirs in
+feather_oracle.c): ``decode_np``, ``gemv_f64_np``, ``attention_f64_np`` are the textbook
+reductions the C oracle is pinned against; ``attention_varlen_f64_np`` (build-defined: the
+reference has no variable-length or causal attention) is pinned by reduction to
+``attention_f64_np`` per sequence and by the prefix property of the causal mask;
+``paged_cache_write_np`` (build-defined) by gathering back through the block table.
 """
 from __future__ import annotations
 

@@ -1,7 +1,9 @@
 """numpy restatement of the packed decode step (csrc/decode_step.hip) for the tests.
 TEST INFRASTRUCTURE ONLY.  The step is build-defined (the reference has no model code);
 this file fixes its meaning: float32 element-wise math, every GEMV operand rounded
-fp32 -> fp16 -> FP8 (RNE) and decoded with the kernel decode, GEMV sums in float64."""
+fp32 -> fp16 -> FP8 (RNE) and decoded with the kernel decode, GEMV sums in float64.
+Parity status: the pieces (quant, rmsnorm, rope, online_attention) are pinned by closed forms
+in tests/test_oracle.py; the composition has no external reference: parity unpinned."""
 from __future__ import annotations
 
 import numpy as np

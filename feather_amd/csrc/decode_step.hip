@@ -8,7 +8,8 @@
 //     paged attention                            feather_paged_attn_fp8
 //     o = W_o attn (attention emits packed FP8)  batched GEMV
 //     (h += o) -> RMSNorm -> pack                add_rmsnorm_pack_kernel
-//     gu = W_gate_up x ; silu(g) * u -> pack     batched GEMV, swiglu_pack_kernel
+//     act = pack(silu(W_gate x) * (W_up x))      batched GEMV with the SwiGLU epilogue
+//                                                (or GEMV + swiglu_pack_kernel for odd shapes)
 //     down = W_down act                          batched GEMV (added to h by the next norm)
 // and a final norm + lm_head GEMV.  Every activation that feeds a GEMV is
 // rounded fp32 -> fp16 -> FP8 (RNE, as pack_fp8_tensor does) and packed four
@@ -205,7 +206,8 @@ static int plan_splits(int64_t M, int64_t K) {
 struct StepPlan {
     int s_qkv, s_o, s_gu, s_down;
     int64_t qkv_rows;
-    size_t b_h, b_delta, b_xq, b_qkv, b_qp, b_gu, b_ctx;
+    bool fused_mlp;                              // gate/up GEMV with the SwiGLU epilogue (no fp32 gate/up buffer)
+    size_t b_h, b_delta, b_xq, b_act, b_qkv, b_qp, b_gu, b_ctx;
 };
 
 static StepPlan plan_step(const feather_decoder_t *dec, int64_t batch) {
@@ -214,15 +216,17 @@ static StepPlan plan_step(const feather_decoder_t *dec, int64_t batch) {
     P.qkv_rows = (nq + 2 * nkv) * d;
     P.s_qkv = plan_splits(P.qkv_rows, H);
     P.s_o = plan_splits(H, nq * d);
-    P.s_gu = plan_splits(2 * I, H);
+    P.fused_mlp = H % 256 == 0 && I % 4 == 0;
+    P.s_gu = P.fused_mlp ? 1 : plan_splits(2 * I, H);
     P.s_down = plan_splits(H, I);
     auto up = [](int64_t b) { return (size_t)((b + 255) / 256 * 256); };
     P.b_h = up(batch * H * 4);
     P.b_delta = up((int64_t)(P.s_o > P.s_down ? P.s_o : P.s_down) * batch * H * 4);
     P.b_xq = up(batch * (H > I ? H : I));
+    P.b_act = up(batch * I);
     P.b_qkv = up((int64_t)P.s_qkv * batch * P.qkv_rows * 4);
     P.b_qp = up(batch * nq * d);
-    P.b_gu = up((int64_t)P.s_gu * batch * 2 * I * 4);
+    P.b_gu = P.fused_mlp ? 0 : up((int64_t)P.s_gu * batch * 2 * I * 4);
     P.b_ctx = up(batch * 4);
     return P;
 }
@@ -239,6 +243,7 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
     float *h = (float *)take(P.b_h);
     float *delta = (float *)take(P.b_delta);
     uint32_t *xq = (uint32_t *)take(P.b_xq);
+    uint32_t *act = (uint32_t *)take(P.b_act);
     float *qkv = (float *)take(P.b_qkv);
     uint32_t *qp = (uint32_t *)take(P.b_qp);
     float *gu = (float *)take(P.b_gu);
@@ -249,16 +254,17 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
     void *st = (void *)s;
     int rc;
     // out receives `splits` partial results of [batch, M], batch * M floats apart
-    auto gemv = [&](const void *w, float *out, int M, int K, int splits) {
-        if (K % 256 != 0) return feather_gemv_fp8_batched(w, xq, out, M, K, batch, MODE, st);
+    auto gemv_x = [&](const void *w, const uint32_t *x, float *out, int M, int K, int splits) {
+        if (K % 256 != 0) return feather_gemv_fp8_batched(w, x, out, M, K, batch, MODE, st);
         int got = 0;
-        int r = gemv_batched_launch(w, xq, out, M, K, batch, MODE, splits, (int64_t)batch * M, &got, s);
+        int r = gemv_batched_launch(w, x, out, M, K, batch, MODE, splits, (int64_t)batch * M, &got, s);
         if (r == FEATHER_OK && got != splits) {
             set_error("feather_decode_step: GEMV slice plan mismatch (%d vs %d)", got, splits);
             return (int)FEATHER_EINVAL;
         }
         return r;
     };
+    auto gemv = [&](const void *w, float *out, int M, int K, int splits) { return gemv_x(w, xq, out, M, K, splits); };
 #define DS_CHECK(call)            \
     do {                          \
         rc = (call);              \
@@ -287,12 +293,16 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
         hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, delta, P.s_o, hs,
                            L.norm_mlp, xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
-        DS_CHECK(gemv(L.w_gate_up, gu, 2 * I, H, P.s_gu));
-        int64_t items = (int64_t)batch * I / 4;
-        hipLaunchKernelGGL((swiglu_pack_kernel<MODE>), dim3((unsigned)((items + kDsThreads - 1) / kDsThreads)),
-                           dim3(kDsThreads), 0, s, gu, P.s_gu, (int64_t)batch * 2 * I, xq, I, batch);
-        DS_CHECK(check_launch("feather_decode_step (swiglu)"));
-        DS_CHECK(gemv(L.w_down, delta, H, I, P.s_down));
+        if (P.fused_mlp) {
+            DS_CHECK(gemv_batched_swiglu_launch(L.w_gate_up, xq, act, I, H, batch, MODE, s));
+        } else {
+            DS_CHECK(gemv(L.w_gate_up, gu, 2 * I, H, P.s_gu));
+            int64_t items = (int64_t)batch * I / 4;
+            hipLaunchKernelGGL((swiglu_pack_kernel<MODE>), dim3((unsigned)((items + kDsThreads - 1) / kDsThreads)),
+                               dim3(kDsThreads), 0, s, gu, P.s_gu, (int64_t)batch * 2 * I, act, I, batch);
+            DS_CHECK(check_launch("feather_decode_step (swiglu)"));
+        }
+        DS_CHECK(gemv_x(L.w_down, act, delta, H, I, P.s_down));
         pending = delta;
     }
     hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending, P.s_down, hs,
@@ -306,7 +316,7 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
 static int64_t step_scratch_bytes(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx) {
     const StepPlan P = plan_step(dec, batch);
     auto up = [](int64_t b) { return (b + 255) / 256 * 256; };
-    return (int64_t)(P.b_h + P.b_delta + P.b_xq + P.b_qkv + P.b_qp + P.b_gu + P.b_ctx) +
+    return (int64_t)(P.b_h + P.b_delta + P.b_xq + P.b_act + P.b_qkv + P.b_qp + P.b_gu + P.b_ctx) +
            up(feather_paged_attn_scratch_bytes(batch, dec->n_q_heads, dec->head_dim, max_ctx));
 }
 

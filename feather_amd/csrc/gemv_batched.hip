@@ -41,16 +41,22 @@ __device__ __forceinline__ half8_t bg_dec8(uint32_t w0, uint32_t w1) {
 
 // K % 256 == 0, w and x 16-byte aligned.  NB = number of 16-vector column blocks.
 // grid = (row tiles, K slices); slice s covers chunks [s * cps, min((s + 1) * cps, K / 256)).
-template <int MODE, int NB>
+// SWIGLU: W is [gate rows; up rows] (M = 2 * inter); a wave takes 8 gate rows and the 8 up rows
+// of the same indices, and the epilogue writes pack(fp16(silu(gate) * up)) as FP8 words to
+// `packed` ([nvec, inter / 4]) instead of fp32 sums to `out` (one K slice only).
+template <int MODE, int NB, bool SWIGLU>
 __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t *__restrict__ w,
                                                                  const uint8_t *__restrict__ x,
                                                                  float *__restrict__ out, int M, int K, int nvec,
-                                                                 int cps, int64_t part_stride) {
+                                                                 int cps, int64_t part_stride,
+                                                                 uint32_t *__restrict__ packed) {
     extern __shared__ __attribute__((aligned(16))) _Float16 xs[];   // [2][16 * NB][kBgPitch]
     const int lane = threadIdx.x & 63, wave = wave_id();
     const int j = lane & 15, kb = lane >> 4;
     const int row0 = blockIdx.x * kBgRows + 16 * wave;
-    const int row = min(row0 + j, M - 1);
+    const int inter = M / 2;
+    const int g0 = blockIdx.x * (kBgRows / 2) + 8 * wave;        // SWIGLU: first of this wave's 8 gate rows
+    const int row = SWIGLU ? (j < 8 ? min(g0 + j, inter - 1) : inter + min(g0 + j - 8, inter - 1)) : min(row0 + j, M - 1);
     const int n_chunks = K / kBgChunk;
     const int c_begin = blockIdx.y * cps, c_end = min(c_begin + cps, n_chunks);
     const uint8_t *wp = w + (int64_t)row * K + 16 * kb;
@@ -121,6 +127,23 @@ __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t 
         __syncthreads();
         mac(buf, wa);
     }
+    if constexpr (SWIGLU) {
+        // accumulator rows 4 kb + {0..3}: kb 0, 1 hold gate rows g0 + 4 kb + i, kb 2, 3 the up rows of
+        // the same indices, 32 lanes further on
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            float u[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) u[i] = __shfl_xor(acc[nb][i], 32, kWave);
+            const int vec = 16 * nb + j, g = g0 + 4 * kb;
+            if (kb < 2 && vec < nvec && g < inter) {
+                auto f = [](float a, float b) { return a / (1.0f + expf(-a)) * b; };
+                packed[(int64_t)vec * (inter / 4) + g / 4] =
+                    quant4<MODE>(f(acc[nb][0], u[0]), f(acc[nb][1], u[1]), f(acc[nb][2], u[2]), f(acc[nb][3], u[3]));
+            }
+        }
+        return;
+    }
     float *o_base = out + (int64_t)blockIdx.y * part_stride;
     const int r = row0 + 4 * kb;                   // accumulator rows 4 kb + {0..3}, column = vector
 #pragma unroll
@@ -139,20 +162,21 @@ __global__ __launch_bounds__(kBgThreads) void gemv_batched_kernel(const uint8_t 
     }
 }
 
-template <int MODE, int NB>
+template <int MODE, int NB, bool SWIGLU>
 static void bg_launch(const void *w, const void *x, float *out, int M, int K, int nvec, int splits, int cps,
-                      int64_t part_stride, hipStream_t s) {
+                      int64_t part_stride, uint32_t *packed, hipStream_t s) {
     const size_t lds = (size_t)2 * 16 * NB * kBgPitch * sizeof(_Float16);
     if (lds > 64 * 1024) {
         static bool raised = false;                // once per process: allow more than 64 KB of dynamic LDS
         if (!raised) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_batched_kernel<MODE, NB>),
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_batched_kernel<MODE, NB, SWIGLU>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             raised = true;
         }
     }
-    hipLaunchKernelGGL((gemv_batched_kernel<MODE, NB>), dim3((unsigned)((M + kBgRows - 1) / kBgRows), (unsigned)splits),
-                       dim3(kBgThreads), lds, s, (const uint8_t *)w, (const uint8_t *)x, out, M, K, nvec, cps, part_stride);
+    hipLaunchKernelGGL((gemv_batched_kernel<MODE, NB, SWIGLU>), dim3((unsigned)((M + kBgRows - 1) / kBgRows), (unsigned)splits),
+                       dim3(kBgThreads), lds, s, (const uint8_t *)w, (const uint8_t *)x, out, M, K, nvec, cps, part_stride,
+                       packed);
 }
 
 int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M, int64_t K, int64_t nvec, int mode,
@@ -163,7 +187,7 @@ int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M,
     splits = (n_chunks + cps - 1) / cps;           // no empty slice
     if (splits_out) *splits_out = splits;
     const int nb = (int)((nvec + 15) / 16);
-#define FEATHER_BG(MM, NBB) bg_launch<MM, NBB>(w, x, out_f32, (int)M, (int)K, (int)nvec, splits, cps, part_stride, stream)
+#define FEATHER_BG(MM, NBB) bg_launch<MM, NBB, false>(w, x, out_f32, (int)M, (int)K, (int)nvec, splits, cps, part_stride, nullptr, stream)
     if (mode == FEATHER_E5M2) {
         switch (nb) { case 1: FEATHER_BG(FEATHER_E5M2, 1); break; case 2: FEATHER_BG(FEATHER_E5M2, 2); break;
                       case 3: FEATHER_BG(FEATHER_E5M2, 3); break; default: FEATHER_BG(FEATHER_E5M2, 4); }
@@ -173,6 +197,25 @@ int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M,
     }
 #undef FEATHER_BG
     return check_launch("feather_gemv_fp8_batched");
+}
+
+// act = pack(fp16(silu(W_gate x) * (W_up x))) with w = [gate rows; up rows] ([2 * inter, K]); the
+// GEMV and the activation in one kernel, no fp32 round trip.  Needs K % 256 == 0, inter % 4 == 0.
+int gemv_batched_swiglu_launch(const void *w, const void *x, uint32_t *act_packed, int64_t inter, int64_t K,
+                               int64_t nvec, int mode, hipStream_t stream) {
+    const int n_chunks = (int)(K / kBgChunk);
+    const int nb = (int)((nvec + 15) / 16);
+#define FEATHER_BG(MM, NBB) \
+    bg_launch<MM, NBB, true>(w, x, nullptr, (int)(2 * inter), (int)K, (int)nvec, 1, n_chunks, 0, act_packed, stream)
+    if (mode == FEATHER_E5M2) {
+        switch (nb) { case 1: FEATHER_BG(FEATHER_E5M2, 1); break; case 2: FEATHER_BG(FEATHER_E5M2, 2); break;
+                      case 3: FEATHER_BG(FEATHER_E5M2, 3); break; default: FEATHER_BG(FEATHER_E5M2, 4); }
+    } else {
+        switch (nb) { case 1: FEATHER_BG(FEATHER_E4M3, 1); break; case 2: FEATHER_BG(FEATHER_E4M3, 2); break;
+                      case 3: FEATHER_BG(FEATHER_E4M3, 3); break; default: FEATHER_BG(FEATHER_E4M3, 4); }
+    }
+#undef FEATHER_BG
+    return check_launch("feather_decode_step (gate_up + swiglu)");
 }
 
 }  // namespace feather

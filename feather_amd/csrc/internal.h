@@ -22,4 +22,10 @@ int paged_attn_launch(const void *q, const void *k_cache, const void *v_cache, c
 int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M, int64_t K, int64_t nvec, int mode,
                         int splits, int64_t part_stride, int *splits_out, hipStream_t stream);
 
+// As gemv_batched_launch for w = [gate rows; up rows] ([2 * inter, K]) with the SwiGLU activation
+// and the FP8 quantisation fused: act_packed [nvec, inter / 4] words.  Needs K % 256 == 0,
+// inter % 4 == 0, 16-byte aligned w and x.
+int gemv_batched_swiglu_launch(const void *w, const void *x, uint32_t *act_packed, int64_t inter, int64_t K,
+                               int64_t nvec, int mode, hipStream_t stream);
+
 }  // namespace feather

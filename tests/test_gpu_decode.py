@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("mode,hidden,nq,nkv,inter", [("E4M3", 512, 8, 2, 1024), ("E5M2", 256, 4, 4, 512),
-                                                      ("E4M3", 1024, 16, 1, 1536)])
+                                                      ("E4M3", 1024, 16, 1, 1536), ("E4M3", 320, 5, 1, 704)])
 def test_decode_step_vs_oracle(orc, mode, hidden, nq, nkv, inter):
     from feather_amd.routines.decode import DecoderConfig, PackedDecoder, random_weights
     from oracle import decode_ref

@@ -22,6 +22,11 @@
 // accumulated by one more MFMA per step whose A operand is a constant block of
 // ones, so they cost no vector-ALU work.
 //
+// E5M2 is the matrix core's bf8 operand format, so in that mode S^T runs on
+// v_mfma_f32_16x16x32_bf8_bf8 straight from the packed K and Q bytes (no decode
+// of K, half the LDS bytes, twice the MFMA rate); the products are the same
+// exact fp16 x fp16 products, accumulated in fp32.
+//
 // Numerics follow the reference kernel (feather/routines/attention.py:24-108):
 // fp16 x fp16 products accumulated in fp32, scores scaled in fp32, online
 // softmax in fp32 (computed as 2^x with log2(e) folded into the scale), P
@@ -70,7 +75,12 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
     int keys_scored, int mask_tail, const int32_t *__restrict__ cu_seqlens, int tiles_per_seq, int total_rows,
     int causal) {
     constexpr int DW = D / 4;              // packed words per row
-    constexpr int KS = D + 8;              // fp16 per K row in LDS (16 B pad against bank conflicts)
+    // E5M2 codes ARE the bf8 operand format of the matrix core: the score product runs on
+    // v_mfma_f32_16x16x32_bf8_bf8 straight from the packed bytes (exact products, fp32 accumulation,
+    // twice the fp16 MFMA rate, no decode, half the LDS bytes for K); V still goes through fp16
+    // because P is an fp16 operand (the reference rounds P to fp16, attention.py:90).
+    constexpr bool BF8 = MODE == FEATHER_E5M2;
+    constexpr int KS = BF8 ? (D + 16) / 2 : D + 8;   // K row pitch in LDS, in fp16 units (bf8: D + 16 bytes)
     constexpr int VS = BN;                 // fp16 per V^T row in LDS (16-byte chunks XOR-swizzled by row)
     constexpr int CH = BN / 8;             // 16-byte chunks per V^T row
     constexpr int QT = 64 * QB;            // queries per workgroup
@@ -120,7 +130,8 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
     const uint32_t *vh = v + kv_row0 * DW;
 
     // ---- Q fragments (B operand of S^T), resident in registers
-    half8_t qf[QB][STEPS];
+    half8_t qf[BF8 ? 1 : QB][BF8 ? 1 : STEPS];
+    long qf8[BF8 ? QB : 1][BF8 ? STEPS : 1];   // bf8: the raw 8 codes
 #pragma unroll
     for (int b = 0; b < QB; b++) {
         int row = q0 + 16 * b + j;
@@ -128,7 +139,8 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
         for (int s = 0; s < STEPS; s++) {
             u32x2 w = u32x2{0, 0};
             if (row < L) w = *reinterpret_cast<const u32x2 *>(qh + (int64_t)row * DW + 8 * s + 2 * kb);
-            qf[b][s] = dec8<MODE>(w.x, w.y);
+            if constexpr (BF8) qf8[b][s] = __builtin_bit_cast(long, w);
+            else qf[b][s] = dec8<MODE>(w.x, w.y);
         }
     }
 
@@ -174,10 +186,14 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
             int u = tid + kAttnThreads * i;
             // K: 16 codes of one key -> 16 fp16, row-major [key][d]
             int key = u / (D / 16), c16 = u % (D / 16);
-            half8_t lo = dec8<MODE>(kreg[i].x, kreg[i].y), hi = dec8<MODE>(kreg[i].z, kreg[i].w);
-            half8_t *kd = reinterpret_cast<half8_t *>(k_lds + key * KS + 16 * c16);
-            kd[0] = lo;
-            kd[1] = hi;
+            if constexpr (BF8) {
+                *reinterpret_cast<u32x4 *>(reinterpret_cast<unsigned char *>(k_lds) + key * (2 * KS) + 16 * c16) = kreg[i];
+            } else {
+                half8_t lo = dec8<MODE>(kreg[i].x, kreg[i].y), hi = dec8<MODE>(kreg[i].z, kreg[i].w);
+                half8_t *kd = reinterpret_cast<half8_t *>(k_lds + key * KS + 16 * c16);
+                kd[0] = lo;
+                kd[1] = hi;
+            }
             // V: 4 keys x 4 dims -> V^T[dd][pos], key order permuted inside each
             // group of 32 so that slot (kb, 4a + r) holds key 16a + 4kb + r
             int ddw = u % DW, kg = u / DW;
@@ -243,10 +259,19 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
             for (int c = 0; c < KB16; c++) {
 #pragma unroll
                 for (int st = 0; st < STEPS; st++) {
-                    half8_t kf = *reinterpret_cast<const half8_t *>(k_lds + (16 * c + j) * KS + 32 * st + 8 * kb);
+                    if constexpr (BF8) {
+                        const long kf = *reinterpret_cast<const long *>(reinterpret_cast<const unsigned char *>(k_lds) +
+                                                                       (16 * c + j) * (2 * KS) + 32 * st + 8 * kb);
 #pragma unroll
-                    for (int b = 0; b < SB; b++)
-                        s[b][c] = mfma16(kf, qf[b0 + b][st], st == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : s[b][c]);
+                        for (int b = 0; b < SB; b++)
+                            s[b][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(
+                                kf, qf8[b0 + b][st], st == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : s[b][c], 0, 0, 0);
+                    } else {
+                        half8_t kf = *reinterpret_cast<const half8_t *>(k_lds + (16 * c + j) * KS + 32 * st + 8 * kb);
+#pragma unroll
+                        for (int b = 0; b < SB; b++)
+                            s[b][c] = mfma16(kf, qf[b0 + b][st], st == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : s[b][c]);
+                    }
                 }
             }
             // ---- online softmax, one query per lane column.  The running maximum is kept on
@@ -342,7 +367,8 @@ struct AttnArgs {
 template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC>
 static int launch_attn(const AttnArgs &a, hipStream_t s) {
     constexpr int QT = 64 * QB;
-    constexpr size_t lds = (size_t)(BN * (D + 8) + D * BN) * 2 * 2;  // two (K, V^T) buffers
+    constexpr int KS = MODE == FEATHER_E5M2 ? (D + 16) / 2 : D + 8;   // K row pitch in fp16 units, as in the kernel
+    constexpr size_t lds = (size_t)(BN * KS + D * BN) * 2 * 2;        // two (K, V^T) buffers
     const int64_t L = VC ? a.max_seqlen : a.L;
     const int tiles_per_seq = (int)((L + QT - 1) / QT);
     const int64_t tiles = VC ? tiles_per_seq * a.n_seq : tiles_per_seq;

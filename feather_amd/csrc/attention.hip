@@ -400,7 +400,7 @@ static int launch_attn(const AttnArgs &a, hipStream_t s) {
 template <int MODE, bool VC>
 static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
     switch (d) {
-        case 64: return launch_attn<64, MODE, 4, 2, 64, 2, VC>(a, s);
+        case 64: return launch_attn<64, MODE, 4, 4, 64, 2, VC>(a, s);   // all four query blocks share every K fragment
         case 128: return launch_attn<128, MODE, 2, 2, 64, 2, VC>(a, s);
         case 256: return launch_attn<256, MODE, 1, 1, 32, 1, VC>(a, s);
         case 512: return launch_attn<512, MODE, 1, 1, 32, 1, VC>(a, s);

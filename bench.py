@@ -194,6 +194,18 @@ def main() -> int:
                                       10, 2, sync)
                 extra[f"sdpa_causal_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
             del qkv16, pk
+        # wide heads: B1 H8, d = 256 / 512, E4M3, vs fp16 SDPA
+        for d, L in ((256, 1024), (256, 4096), (256, 8192), (512, 1024), (512, 4096), (512, 8192)):
+            B, H = 1, 8
+            qkv16 = [randn(B, H, L, d).half() for _ in range(3)]
+            pk = [feather.pack_fp8_tensor(t, mode="E4M3").view(B, H, L, d // 4) for t in qkv16]
+            us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
+                                                                                mode="E4M3"), 10, 3, sync)
+            extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_us"] = round(us, 1)
+            extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_TFLOPs"] = round(4.0 * B * H * L * L * d / us / 1e6, 1)
+            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 3, sync)
+            extra[f"sdpa_fp16_b1h8_d{d}_L{L}_us"] = round(us_sdpa, 1)
+            del qkv16, pk
         torch.cuda.empty_cache()
         # paged-attention decode, 32 sequences x 32 query heads over 4 KV heads, d=64, E4M3, blocks of 16
         # tokens scattered by a random block table; bytes = K and V codes of every context token once

@@ -1,12 +1,12 @@
 // Flash-attention forward on FP8-packed Q/K/V (prefill): fixed-length heads, or variable-length
 // sequences packed back to back with an optional causal mask.
 //
-// Work split.  One workgroup (4 waves) owns a tile of 64*QB queries of one
-// head; each wave owns 16*QB of them for the whole key loop.  Keys/values are
+// Work split.  One workgroup (WAVES waves, 4 or 8) owns a tile of 16*QB*WAVES
+// queries of one head; each wave owns 16*QB of them for the whole key loop.  Keys/values are
 // streamed in tiles of BN keys: the PACKED tile is fetched from global memory
 // into registers one tile ahead (so HBM/L2 latency overlaps the MFMA work of
 // the current tile), decoded to fp16 on its way into LDS, and read from LDS as
-// MFMA operands by all four waves.
+// MFMA operands by every wave.
 //
 // Matrix cores.  Everything is computed transposed so that one lane keeps one
 // query for the whole kernel:
@@ -37,8 +37,6 @@
 
 namespace feather {
 
-constexpr int kAttnThreads = 256;
-
 __device__ __forceinline__ float4_t mfma16(half8_t a, half8_t b, float4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
@@ -59,7 +57,7 @@ __device__ __forceinline__ float xor_lane(float x, int mask) {
     return __shfl_xor(x, mask, kWave);
 }
 
-// QB  16-query blocks per wave (a workgroup owns 64 * QB queries)
+// QB  16-query blocks per wave (a workgroup owns 16 * QB * WAVES queries)
 // SB  query blocks scored together (SB divides QB)
 // BN  keys per tile
 // OCC workgroups per CU the register budget is sized for (2 keeps every MFMA
@@ -68,8 +66,8 @@ __device__ __forceinline__ float xor_lane(float x, int mask) {
 //     cu_seqlens (n_seq + 1 row offsets) occupies rows [cu[s], cu[s+1]) of every head and
 //     attends only to itself; with causal != 0 query i sees keys 0..i of its sequence.
 //     tiles_per_head = n_seq * tiles_per_seq; L, keys_scored and mask_tail are not used.
-template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC>
-__global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
+template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC, int WAVES = 4>
+__global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     const uint32_t *__restrict__ q, const uint32_t *__restrict__ k, const uint32_t *__restrict__ v,
     float *__restrict__ out, int L, int n_heads, int kv_group, int tiles_per_head, float scale_log2e,
     int keys_scored, int mask_tail, const int32_t *__restrict__ cu_seqlens, int tiles_per_seq, int total_rows,
@@ -83,9 +81,10 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
     constexpr int KS = BF8 ? (D + 16) / 2 : D + 8;   // K row pitch in LDS, in fp16 units (bf8: D + 16 bytes)
     constexpr int VS = BN;                 // fp16 per V^T row in LDS (16-byte chunks XOR-swizzled by row)
     constexpr int CH = BN / 8;             // 16-byte chunks per V^T row
-    constexpr int QT = 64 * QB;            // queries per workgroup
+    constexpr int kAttnThreads = 64 * WAVES;
+    constexpr int QT = 16 * QB * WAVES;    // queries per workgroup
     constexpr int NU = BN * D / 16 / kAttnThreads;  // 16-code units per thread per tile
-    static_assert(NU >= 1, "tile too small for 256 threads");
+    static_assert(NU >= 1, "tile too small for the workgroup");
     constexpr int KB16 = BN / 16, KB32 = BN / 32, DB = D / 16, STEPS = D / 32;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -113,11 +112,11 @@ __global__ __launch_bounds__(kAttnThreads, OCC) void flash_attn_kernel(
         if (causal) tile = tiles_per_seq - 1 - tile;          // the tiles with the longest key loops start first
         const int r0 = cu_seqlens[seq];
         L = cu_seqlens[seq + 1] - r0;
-        if (tile * (64 * QB) >= L) return;                    // past the end of this sequence (whole workgroup)
+        if (tile * QT >= L) return;                    // past the end of this sequence (whole workgroup)
         q_row0 = (int64_t)head * total_rows + r0;
         kv_row0 = (int64_t)kv_head * total_rows + r0;
         mask_tail = 1;
-        const int last_key = causal ? min(L, (tile + 1) * (64 * QB)) : L;
+        const int last_key = causal ? min(L, (tile + 1) * QT) : L;
         keys_scored = (last_key + BN - 1) / BN * BN;
     }
 
@@ -364,9 +363,9 @@ struct AttnArgs {
     int causal;
 };
 
-template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC>
+template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC, int WAVES = 4>
 static int launch_attn(const AttnArgs &a, hipStream_t s) {
-    constexpr int QT = 64 * QB;
+    constexpr int QT = 16 * QB * WAVES;
     constexpr int KS = MODE == FEATHER_E5M2 ? (D + 16) / 2 : D + 8;   // K row pitch in fp16 units, as in the kernel
     constexpr size_t lds = (size_t)(BN * KS + D * BN) * 2 * 2;        // two (K, V^T) buffers
     const int64_t L = VC ? a.max_seqlen : a.L;
@@ -377,7 +376,7 @@ static int launch_attn(const AttnArgs &a, hipStream_t s) {
     if (blocks == 0) return FEATHER_OK;
     // the reference scores whole 64-key tiles (zero rows past L); otherwise only tiles of BN up to L
     int64_t keys_scored = a.tail == FEATHER_TAIL_REFERENCE ? (L + 63) / 64 * 64 : (L + BN - 1) / BN * BN;
-    auto kern = flash_attn_kernel<D, MODE, QB, SB, BN, OCC, VC>;
+    auto kern = flash_attn_kernel<D, MODE, QB, SB, BN, OCC, VC, WAVES>;
     if (lds > 64 * 1024) {
         static bool attr_set = false;  // per instantiation
         if (!attr_set) {
@@ -389,7 +388,7 @@ static int launch_attn(const AttnArgs &a, hipStream_t s) {
         }
     }
     const float log2e = 1.4426950408889634f;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kAttnThreads), lds, s, (const uint32_t *)a.q,
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * WAVES), lds, s, (const uint32_t *)a.q,
                        (const uint32_t *)a.k, (const uint32_t *)a.v, (float *)a.out, (int)L, (int)a.n_heads,
                        (int)a.kv_group, (int)tiles, a.scale * log2e, (int)keys_scored,
                        a.tail == FEATHER_TAIL_MASK ? 1 : 0, (const int32_t *)a.cu_seqlens, tiles_per_seq,
@@ -397,13 +396,26 @@ static int launch_attn(const AttnArgs &a, hipStream_t s) {
     return check_launch("feather_flash_attn_fp8");
 }
 
+// Workgroup shapes.  d = 64 keeps four waves of 64 queries each.  From d = 128 on, decoding a K/V
+// tile into LDS is a large share of a workgroup's vector work, so eight waves (twice the queries per
+// staged tile, two waves per SIMD to overlap the barrier-separated phases) are faster wherever the
+// coarser grid still covers the chip's 256 CUs; d = 256 takes eight waves and 64-key tiles at every
+// length (four independent score chains per wave instead of two).
 template <int MODE, bool VC>
 static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
+    const int64_t rows = VC ? a.max_seqlen : a.L, seqs = VC ? a.n_seq : 1;
+    auto fills_chip = [&](int64_t queries_per_group) {
+        return (rows + queries_per_group - 1) / queries_per_group * seqs * a.n_heads >= 256;
+    };
     switch (d) {
         case 64: return launch_attn<64, MODE, 4, 4, 64, 2, VC>(a, s);   // all four query blocks share every K fragment
-        case 128: return launch_attn<128, MODE, 2, 2, 64, 2, VC>(a, s);
-        case 256: return launch_attn<256, MODE, 1, 1, 32, 1, VC>(a, s);
-        case 512: return launch_attn<512, MODE, 1, 1, 32, 1, VC>(a, s);
+        case 128:
+            if (fills_chip(256)) return launch_attn<128, MODE, 2, 2, 64, 1, VC, 8>(a, s);
+            return launch_attn<128, MODE, 2, 2, 64, 2, VC>(a, s);
+        case 256: return launch_attn<256, MODE, 1, 1, 64, 1, VC, 8>(a, s);
+        case 512:
+            if (fills_chip(128)) return launch_attn<512, MODE, 1, 1, 32, 1, VC, 8>(a, s);
+            return launch_attn<512, MODE, 1, 1, 32, 1, VC>(a, s);
     }
     set_error("feather_flash_attn_fp8: head dim %lld not supported (64, 128, 256, 512)", (long long)d);
     return FEATHER_ESHAPE;

@@ -102,6 +102,26 @@ def test_flash_attention_invariants_and_gqa(dev, orc):
     assert torch.equal(grouped, rep)
 
 
+@pytest.mark.parametrize("d", [64, 128])
+def test_flash_attention_e5m2_subnormal_codes_count(dev, orc, d):
+    """E5M2 scores must keep subnormal codes exact: keys of code 0x01 (2^-16) against queries of
+    code 0x7B (57344) give a raw score of 0.875 * d, against 0 for the zero keys;
+    flushing the subnormals would leave a uniform softmax (output -0.5 instead of ~1)."""
+    from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
+    L = 64
+    K = np.zeros((L, d), np.uint8)
+    K[:32] = 0x01
+    Q = np.full((L, d), 0x7B, np.uint8)
+    V = np.zeros((L, d), np.uint8)
+    V[:32], V[32:] = 0x3C, 0xC0  # 1.0 and -2.0
+    q, k, v = (np.ascontiguousarray(a).view(np.uint32) for a in (Q, K, V))
+    out = flash_attention_fp8_acc_fp32_gpu(_dev_words(q, dev), _dev_words(k, dev), _dev_words(v, dev), L, d // 4,
+                                           mode="E5M2").cpu().numpy()
+    want = orc.attention_f64_np(q, k, v, L, d, "E5M2")[0]
+    assert want[0, 0] > 0.9
+    assert np.abs(out - want).max() <= 1e-5
+
+
 def test_flash_attention_config_sized_property(dev):
     """B4 H16 L4096 d64 E5M2: too big for the scalar oracle; compare with torch SDPA (fp32
     math) of the decoded operands on device and check determinism."""
@@ -124,6 +144,9 @@ def test_flash_attention_config_sized_property(dev):
 @pytest.mark.parametrize("mode,B,H,L,d,causal", [
     ("E5M2", 4, 16, 8192, 64, False), ("E4M3", 1, 8, 4096, 256, False), ("E4M3", 1, 8, 8192, 512, False),
     ("E4M3", 1, 8, 1024, 256, True), ("E5M2", 2, 4, 8192, 64, True),
+    # eight-wave workgroups: d = 128 and d = 512 switch to them once the coarser grid covers 256 CUs
+    ("E5M2", 4, 16, 4096, 128, False), ("E4M3", 4, 16, 1024, 128, True), ("E4M3", 1, 8, 4100, 512, True),
+    ("E5M2", 1, 8, 4096, 256, False),
 ])
 def test_flash_attention_full_size_rows_vs_fp32_math(dev, mode, B, H, L, d, causal):
     """The remaining attention shapes of the benchmark configurations, too big for the scalar oracle:
@@ -236,6 +259,8 @@ def test_paged_attention_config_shape(dev, orc):
     ("E5M2", 2, 1, 64, [70, 0, 300, 1], True), ("E5M2", 2, 2, 64, [70, 0, 300, 1], False),
     ("E4M3", 4, 2, 64, [513, 255], True), ("E5M2", 1, 1, 128, [129, 64], True),
     ("E4M3", 1, 1, 256, [100, 37], True), ("E5M2", 1, 1, 512, [65], True), ("E4M3", 2, 1, 128, [200], False),
+    # enough (head, sequence, tile) groups for the eight-wave d = 128 shape; lengths straddle its 256-query tile
+    ("E4M3", 8, 4, 128, [257, 31, 0, 256] * 4, True), ("E5M2", 16, 16, 128, [300, 90] * 4, False),
 ])
 def test_varlen_attention_vs_oracle(dev, orc, mode, n_heads, n_kv, d, lens, causal):
     from feather_amd.routines.attention import flash_attention_fp8_varlen_acc_fp32_gpu

@@ -7,7 +7,11 @@
 // index order.  (A single-kernel "last workgroup finishes" scheme needs
 // device-scope release/acquire around the arrival counter, which on this
 // multi-XCD part costs an L2 write-back/invalidate per workgroup and measured
-// ~45 us for 2^24 elements; the second launch costs a few us.)
+// ~45 us for 2^24 elements; the second launch costs a few us.  The same scheme
+// with relaxed device-scope atomics only (partial published by an exchange,
+// ticket drawn after it returned, partials read back with atomic loads) gives
+// correct sums without fences, but the tickets serialise at the memory side:
+// 22 us with 1024 workgroups, 11-14 us with 256, no better than two launches.)
 #include "common.h"
 
 namespace feather {
@@ -97,14 +101,31 @@ __global__ __launch_bounds__(kDotThreads) void dot_kernel(const uint32_t *__rest
     }
 }
 
-// One wave: lane l adds partials l, l + 64, ... in order, then the wave fold.
-__global__ __launch_bounds__(kWave) void dot_finish_kernel(const uint32_t *__restrict__ scratch,
-                                                          float *__restrict__ out, int n_partials) {
+// One workgroup adds the partials in a fixed order: thread t takes t, t + 256, ... (every load is
+// issued before the first add: a loop of dependent loads pays one memory round trip per turn and
+// made this kernel take 5.7 us for 1024 partials), then the wave fold, then the waves in order.
+constexpr int kFinishThreads = 256;
+__global__ __launch_bounds__(kFinishThreads) void dot_finish_kernel(const uint32_t *__restrict__ scratch,
+                                                                   float *__restrict__ out, int n_partials) {
+    __shared__ float wave_part[kFinishThreads / kWave];
     const float *partials = reinterpret_cast<const float *>(scratch + 16);
+    constexpr int kPer = kDotMaxBlocks / kFinishThreads;
+    float v[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; k++) v[k] = partials[min((int)threadIdx.x + kFinishThreads * k, n_partials - 1)];
     float t = 0.f;
-    for (int i = threadIdx.x; i < n_partials; i += kWave) t += partials[i];
+#pragma unroll
+    for (int k = 0; k < kPer; k++)
+        if ((int)threadIdx.x + kFinishThreads * k < n_partials) t += v[k];
     t = wave_sum(t);
-    if (threadIdx.x == 0) out[0] = t;
+    if (lane_id() == 0) wave_part[wave_id()] = t;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float r = 0.f;
+#pragma unroll
+        for (int w = 0; w < kFinishThreads / kWave; w++) r += wave_part[w];
+        out[0] = r;
+    }
 }
 
 template <int KIND>
@@ -123,7 +144,7 @@ static int launch_dot(const void *x1, const void *x2, void *out, void *scratch, 
                            (const uint32_t *)x1, (const uint32_t *)x2, (float *)out, (uint32_t *)scratch, n_words);
     int rc = check_launch(what);
     if (rc != FEATHER_OK) return rc;
-    hipLaunchKernelGGL(dot_finish_kernel, dim3(1), dim3(kWave), 0, s, (const uint32_t *)scratch, (float *)out,
+    hipLaunchKernelGGL(dot_finish_kernel, dim3(1), dim3(kFinishThreads), 0, s, (const uint32_t *)scratch, (float *)out,
                        (int)blocks);
     return check_launch(what);
 }

@@ -208,14 +208,16 @@ static void bg_launch_kg(const void *w, const void *x, float *out, int M, int K,
                        (const uint8_t *)w, (const uint8_t *)x, out, M, K, nvec, cps, part_stride, packed);
 }
 
-// Two K groups per workgroup wherever every slice (the last one too) gives each group at least two
-// chunks.  Measured at 32 vectors, E4M3: 16384 x 16384 90.7 -> 71.4 us, 11264 x 2048 11.1 -> 9.5 us;
-// four groups (1024 threads) were slower than two on every shape tried.
+// Two K groups per workgroup when every slice (the last one too) gives each group at least two chunks
+// and either the grid does not fill the chip twice over or the K walk is long.  Measured at 32 vectors,
+// E4M3: 16384 x 16384 90.7 -> 71.4 us, 11264 x 2048 11.1 -> 9.5 us, but 32000 x 2048 (500 workgroups of
+// 8 chunks) 18.1 -> 18.7 us; four groups (1024 threads) were slower than two on every shape tried.
 template <int MODE, int NB, bool SWIGLU>
 static void bg_launch(const void *w, const void *x, float *out, int M, int K, int nvec, int splits, int cps,
                       int64_t part_stride, uint32_t *packed, hipStream_t s) {
     const int last = K / kBgChunk - (splits - 1) * cps;   // chunks of the last slice
-    if (cps >= 4 && cps % 2 == 0 && last % 2 == 0)
+    const int64_t groups = (int64_t)((M + kBgRows - 1) / kBgRows) * splits;
+    if (cps >= 4 && cps % 2 == 0 && last % 2 == 0 && (groups <= 256 || cps >= 16))
         bg_launch_kg<MODE, NB, SWIGLU, 2>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);
     else
         bg_launch_kg<MODE, NB, SWIGLU, 1>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);

@@ -19,6 +19,11 @@
 // A wave issues the loads of all its steps (up to four) before it consumes the
 // first, so the dependent chains block id -> row address -> data of the steps
 // overlap instead of adding up.
+// (Letting the last split of a sequence to finish do the merge, with the partials
+// and an arrival counter handled by device-scope atomics, gives the same results
+// without the second launch but was slower: write-through stores, the ticket and
+// the read-back are three memory-side round trips in a row, +7 us per call
+// against ~4 us for the merge kernel.)
 #include "internal.h"
 #include "common.h"
 

@@ -261,6 +261,8 @@ def test_paged_attention_config_shape(dev, orc):
     ("E4M3", 1, 1, 256, [100, 37], True), ("E5M2", 1, 1, 512, [65], True), ("E4M3", 2, 1, 128, [200], False),
     # enough (head, sequence, tile) groups for the eight-wave d = 128 shape; lengths straddle its 256-query tile
     ("E4M3", 8, 4, 128, [257, 31, 0, 256] * 4, True), ("E5M2", 16, 16, 128, [300, 90] * 4, False),
+    # the eight-wave d = 64 shape (non-causal, >= 256 groups of 512 queries), lengths around its tile
+    ("E5M2", 16, 8, 64, [513, 100, 512, 0] * 4, False),
 ])
 def test_varlen_attention_vs_oracle(dev, orc, mode, n_heads, n_kv, d, lens, causal):
     from feather_amd.routines.attention import flash_attention_fp8_varlen_acc_fp32_gpu

@@ -37,6 +37,8 @@ def _qkv(rng, heads, L, d, mode, orc, ints=False):
 @pytest.mark.parametrize("mode,heads,L,d", [
     ("E5M2", 1, 128, 64), ("E5M2", 3, 256, 64), ("E4M3", 2, 128, 64), ("E5M2", 2, 128, 128),
     ("E4M3", 1, 64, 256), ("E4M3", 1, 96, 512), ("E5M2", 1, 64, 512), ("E5M2", 8, 1024, 64),
+    # d = 256 below 256 workgroups: two wave groups split the key tiles (even, odd and ragged tile counts)
+    ("E4M3", 2, 200, 256), ("E5M2", 1, 330, 256), ("E4M3", 1, 128, 256),
 ])
 def test_flash_attention_vs_oracle(dev, orc, mode, heads, L, d):
     from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
@@ -146,7 +148,7 @@ def test_flash_attention_config_sized_property(dev):
     ("E4M3", 1, 8, 1024, 256, True), ("E5M2", 2, 4, 8192, 64, True),
     # eight-wave workgroups: d = 128 and d = 512 switch to them once the coarser grid covers 256 CUs
     ("E5M2", 4, 16, 4096, 128, False), ("E4M3", 4, 16, 1024, 128, True), ("E4M3", 1, 8, 4100, 512, True),
-    ("E5M2", 1, 8, 4096, 256, False),
+    ("E5M2", 1, 8, 4096, 256, False), ("E4M3", 1, 8, 1024, 256, False),
 ])
 def test_flash_attention_full_size_rows_vs_fp32_math(dev, mode, B, H, L, d, causal):
     """The remaining attention shapes of the benchmark configurations, too big for the scalar oracle:
@@ -263,6 +265,7 @@ def test_paged_attention_config_shape(dev, orc):
     ("E4M3", 8, 4, 128, [257, 31, 0, 256] * 4, True), ("E5M2", 16, 16, 128, [300, 90] * 4, False),
     # the eight-wave d = 64 shape (non-causal, >= 256 groups of 512 queries), lengths around its tile
     ("E5M2", 16, 8, 64, [513, 100, 512, 0] * 4, False),
+    ("E4M3", 2, 1, 256, [130, 64, 0, 257], False),           # d = 256 with the key tiles split between wave groups
 ])
 def test_varlen_attention_vs_oracle(dev, orc, mode, n_heads, n_kv, d, lens, causal):
     from feather_amd.routines.attention import flash_attention_fp8_varlen_acc_fp32_gpu

@@ -432,16 +432,10 @@ static int launch_attn(const AttnArgs &a, hipStream_t s) {
     // the reference scores whole 64-key tiles (zero rows past L); otherwise only tiles of BN up to L
     int64_t keys_scored = a.tail == FEATHER_TAIL_REFERENCE ? (L + 63) / 64 * 64 : (L + BN - 1) / BN * BN;
     auto kern = flash_attn_kernel<D, MODE, QB, SB, BN, OCC, VC, WAVES, KSPLIT>;
-    if (lds > 64 * 1024) {
-        static bool attr_set = false;  // per instantiation
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            FEATHER_CHECK(e == hipSuccess, FEATHER_ELAUNCH, "feather_flash_attn_fp8: cannot raise LDS limit: %s",
-                          hipGetErrorString(e));
-            attr_set = true;
-        }
-    }
+    static unsigned long long lds_raised = 0;   // per instantiation, one bit per device
+    hipError_t e = raise_lds_limit(reinterpret_cast<const void *>(kern), lds, lds_raised);
+    FEATHER_CHECK(e == hipSuccess, FEATHER_ELAUNCH, "feather_flash_attn_fp8: cannot raise LDS limit: %s",
+                  hipGetErrorString(e));
     const float log2e = 1.4426950408889634f;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * WAVES), lds, s, (const uint32_t *)a.q,
                        (const uint32_t *)a.k, (const uint32_t *)a.v, (float *)a.out, (int)L, (int)a.n_heads,

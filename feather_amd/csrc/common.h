@@ -42,6 +42,21 @@ inline int check_launch(const char *what) {
 
 inline bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
+// Kernels that ask for more than 64 KB of dynamic LDS need the limit raised once per device (the
+// attribute belongs to the device's copy of the code).  `done` is one bit mask per kernel
+// instantiation, kept by the caller in a function-local static.
+inline hipError_t raise_lds_limit(const void *kernel, size_t bytes, unsigned long long &done) {
+    if (bytes <= 64 * 1024) return hipSuccess;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (done & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) done |= bit;
+    return e;
+}
+
 // ---------------------------------------------------------------- bit casts
 
 __device__ __forceinline__ half2_t as_half2(uint32_t x) { return __builtin_bit_cast(half2_t, x); }

@@ -195,14 +195,8 @@ template <int MODE, int NB, bool SWIGLU, int KG>
 static void bg_launch_kg(const void *w, const void *x, float *out, int M, int K, int nvec, int splits, int cps,
                          int64_t part_stride, uint32_t *packed, hipStream_t s) {
     const size_t lds = (size_t)KG * 2 * 16 * NB * kBgPitch * sizeof(_Float16);
-    if (lds > 64 * 1024) {
-        static bool raised = false;                // once per process: allow more than 64 KB of dynamic LDS
-        if (!raised) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_batched_kernel<MODE, NB, SWIGLU, KG>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            raised = true;
-        }
-    }
+    static unsigned long long lds_raised = 0;      // per instantiation, one bit per device
+    (void)raise_lds_limit(reinterpret_cast<const void *>(&gemv_batched_kernel<MODE, NB, SWIGLU, KG>), lds, lds_raised);
     hipLaunchKernelGGL((gemv_batched_kernel<MODE, NB, SWIGLU, KG>),
                        dim3((unsigned)((M + kBgRows - 1) / kBgRows), (unsigned)splits), dim3(kBgThreads * KG), lds, s,
                        (const uint8_t *)w, (const uint8_t *)x, out, M, K, nvec, cps, part_stride, packed);

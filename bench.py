@@ -172,26 +172,27 @@ def main() -> int:
         del src, words
         del mats["E5M2"], sub, xs
         torch.cuda.empty_cache()
-        # flash attention, B4 H16 d64, E5M2, vs fp16 SDPA on the same GPU
+        # flash attention, B4 H16 d64, E5M2, vs fp16 SDPA on the same GPU (10 warm-up calls each: the
+        # first few milliseconds of a long-kernel series run below the sustained clock)
         for L in (4096, 8192):
             B, H, d = 4, 16, 64
             qkv16 = [randn(B, H, L, d).half() for _ in range(3)]
             pk = [feather.pack_fp8_tensor(t, mode="E5M2").view(B, H, L, d // 4) for t in qkv16]
             us = gpu_time_us(lambda i: feather.flash_attention_fp8_e5m2_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4),
-                             10, 2, sync)
+                             10, 10, sync)
             flops = 4.0 * B * H * L * L * d
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / us / 1e6, 1)
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_mfma_frac"] = round(flops / us / 1e6 / MFMA_PEAK_F16_TFLOPS, 4)
-            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 2, sync)
+            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync)
             extra[f"sdpa_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
             if L == 8192:   # causal prefill (half the flops) vs causal fp16 SDPA
                 us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
-                                                                                    mode="E5M2", causal=True), 10, 2, sync)
+                                                                                    mode="E5M2", causal=True), 10, 10, sync)
                 extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
                 extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / 2 / us / 1e6, 1)
                 us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16, is_causal=True),
-                                      10, 2, sync)
+                                      10, 10, sync)
                 extra[f"sdpa_causal_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
             del qkv16, pk
         # wide heads: B1 H8, d = 256 / 512, E4M3, vs fp16 SDPA
@@ -200,10 +201,10 @@ def main() -> int:
             qkv16 = [randn(B, H, L, d).half() for _ in range(3)]
             pk = [feather.pack_fp8_tensor(t, mode="E4M3").view(B, H, L, d // 4) for t in qkv16]
             us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
-                                                                                mode="E4M3"), 10, 3, sync)
+                                                                                mode="E4M3"), 10, 10, sync)
             extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_us"] = round(us, 1)
             extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_TFLOPs"] = round(4.0 * B * H * L * L * d / us / 1e6, 1)
-            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 3, sync)
+            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync)
             extra[f"sdpa_fp16_b1h8_d{d}_L{L}_us"] = round(us_sdpa, 1)
             del qkv16, pk
         torch.cuda.empty_cache()

@@ -291,12 +291,16 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
 #pragma unroll
             for (int b = 0; b < SB; b++) {
                 if (ragged || diag) {
-                    const int last = diag ? min(L - 1, q0 + 16 * (b0 + b) + j) : L - 1;   // last visible key
+                    int last = diag ? min(L - 1, q0 + 16 * (b0 + b) + j) : L - 1;   // last visible key
+                    // opaque to the optimiser from here on: otherwise the 16 key-index compares below
+                    // are hoisted out of this rarely taken branch and run for every tile
+                    asm volatile("" : "+v"(last));
+                    const int rel = last - key0 - 4 * kb;   // key 16 c + 4 kb + r of the tile is hidden if 16 c + r > rel
 #pragma unroll
                     for (int c = 0; c < KB16; c++)
 #pragma unroll
                         for (int r = 0; r < 4; r++)
-                            if (key0 + 16 * c + 4 * kb + r > last) s[b][c][r] = -INFINITY;
+                            if (16 * c + r > rel) s[b][c][r] = -INFINITY;
                 }
                 float mx = s[b][0][0];
 #pragma unroll

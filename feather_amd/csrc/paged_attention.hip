@@ -242,11 +242,16 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         // online softmax (lane column = query head), log2 domain; only the last step of a split
         // can hold tokens past its end (wave-uniform test)
         if (t0 + kStepTok > t_end) {
+            // token 16 a + 4 kb + r of the step is past the end if 16 a + r >= rel; rel is made opaque
+            // so that this rarely taken branch stays a branch (if-converted, its compares and selects
+            // run in every step)
+            int rel = t_end - t0 - 4 * kb;
+            asm volatile("" : "+v"(rel));
 #pragma unroll
             for (int a = 0; a < 2; a++)
 #pragma unroll
                 for (int r = 0; r < 4; r++)
-                    if (t0 + 16 * a + 4 * kb + r >= t_end) s[a][r] = -INFINITY;
+                    if (16 * a + r >= rel) s[a][r] = -INFINITY;
         }
         float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
                          fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));

@@ -18,7 +18,7 @@
 // permuting the key order in which V^T is written to LDS, so the softmax
 // output feeds the second MFMA straight from registers: no shuffle, no LDS
 // round trip for P.  Row maxima need one exchange across the 4 lanes that
-// share a query (two bpermute steps); the row sums (softmax denominators) are
+// share a query (a row swap and a half-wave swap); the row sums (softmax denominators) are
 // accumulated by one more MFMA per step whose A operand is a constant block of
 // ones, so they cost no vector-ALU work.
 //
@@ -51,10 +51,6 @@ __device__ __forceinline__ half8_t dec8(uint32_t w0, uint32_t w1) {
     dec_word<MODE>(w1, a, b);
     r.z = a; r.w = b;
     return __builtin_bit_cast(half8_t, r);
-}
-
-__device__ __forceinline__ float xor_lane(float x, int mask) {
-    return __shfl_xor(x, mask, kWave);
 }
 
 // QB  16-query blocks per wave (a workgroup owns 16 * QB * WAVES queries)
@@ -307,8 +303,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                 for (int c = 0; c < KB16; c++)
 #pragma unroll
                     for (int r = 0; r < 4; r++) mx = fmaxf(mx, s[b][c][r]);
-                mx = fmaxf(mx, xor_lane(mx, 16));
-                mx = fmaxf(mx, xor_lane(mx, 32));
+                mx = max_xor32(max_xor16(mx));   // over the four lanes that share the query
                 const float m_old = m_run[b0 + b];
                 const float m_new = fmaxf(m_old, mx);
                 const float mc = m_new * scale_log2e;

@@ -215,6 +215,24 @@ __device__ __forceinline__ float wave_sum(float x) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// max(x, x of lane ^ 16) and max(x, x of lane ^ 32) with the gfx950 row / half-wave swaps: one
+// VALU instruction each instead of an LDS permute with six instructions of index arithmetic.
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of the
+// second, v_permlane32_swap the upper half of the first with the lower half of the second; with
+// both operands holding x, every lane then finds x and its partner's x in the two registers.
+// (Inline assembly: the compiler folds the two results of the corresponding builtins into one when
+// both inputs are the same value.  s_nop 1 covers the VALU-write -> permlane-read wait states.)
+__device__ __forceinline__ float max_xor16(float x) {
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float max_xor32(float x) {
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }
 
 // Index of the wave inside its workgroup, marked as wave-uniform: everything derived from it (row

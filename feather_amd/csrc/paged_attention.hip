@@ -255,8 +255,7 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         }
         float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
                          fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+        mx = max_xor32(max_xor16(mx));
         const float m_new = fmaxf(m_run, mx * scale_log2e);      // scale > 0: the maximum commutes with it
         half8_t p8;
         float rs = 0.f;

@@ -171,6 +171,35 @@ def test_flash_attention_full_size_rows_vs_fp32_math(dev, mode, B, H, L, d, caus
         assert err.item() <= TOL
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_varlen_attention_random_shapes(dev, orc, seed):
+    """Seeded random (mode, head dim, head counts, lengths, causal) draws: the launcher picks between
+    four- and eight-wave workgroups and the key-split shape from the grid size, so cover its choices
+    with lengths that land on and around every tile size."""
+    from feather_amd.routines.attention import flash_attention_fp8_varlen_acc_fp32_gpu
+    rng = np.random.default_rng(1000 + seed)
+    mode = ("E5M2", "E4M3")[seed % 2]
+    d = (64, 128, 256, 512)[(seed // 2) % 4]
+    n_kv = int(rng.integers(1, 5))
+    n_heads = n_kv * int(rng.integers(1, 5))
+    edges = np.array([0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513])
+    n_seq = int(rng.integers(1, 7)) if seed % 3 else int(rng.integers(20, 40))
+    lens = [int(x) for x in rng.choice(edges[edges <= (513 if d <= 128 else 257)], size=n_seq)]
+    if max(lens) == 0:
+        lens[0] = 33
+    causal = bool(seed % 4 < 2)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    total = int(cu[-1])
+    q = orc.pack_fp8(rng.standard_normal((n_heads, total, d)).astype(np.float16), mode).reshape(n_heads, total, d // 4)
+    k = orc.pack_fp8(rng.standard_normal((n_kv, total, d)).astype(np.float16), mode).reshape(n_kv, total, d // 4)
+    v = orc.pack_fp8(rng.standard_normal((n_kv, total, d)).astype(np.float16), mode).reshape(n_kv, total, d // 4)
+    out = flash_attention_fp8_varlen_acc_fp32_gpu(_dev_words(q, dev, q.shape), _dev_words(k, dev, k.shape),
+                                                  _dev_words(v, dev, v.shape), torch.from_numpy(cu).to(dev), max(lens),
+                                                  mode=mode, causal=causal).cpu().numpy()
+    want = orc.attention_varlen_f64_np(q, k, v, cu, d, mode, causal=causal)
+    assert np.isfinite(out).all() and _nerr(out, want) <= TOL
+
+
 # ---------------------------------------------------------------- paged decode
 
 @pytest.mark.parametrize("mode,n_seq,Hq,Hkv,d,bs,max_ctx", [

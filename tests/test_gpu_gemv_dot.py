@@ -172,6 +172,34 @@ def test_gemv_batched_decode_shapes_vs_fp64_math(dev, M, K):
     assert ((out.double() - want).abs().max() / want.abs().max()).item() <= TOL
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_gemv_batched_random_shapes(dev, seed):
+    """Seeded random (mode, M, K, nvec) draws against a float64 matmul of the decoded operands on
+    the device: the launcher switches between one and two K groups per workgroup and the
+    per-vector path on K, M and the vector count; codes are raw random bytes (every code occurs,
+    NaN / inf codes of E5M2 masked out)."""
+    import feather_amd as feather
+    from feather_amd.routines.gemv import gemv_fp8_batched_acc_fp32_gpu
+    rng = np.random.default_rng(500 + seed)
+    mode = ("E4M3", "E5M2")[seed % 2]
+    M = int(rng.integers(1, 700))
+    K = int(rng.choice([4, 100, 256, 512, 768, 1024, 1280, 2048, 4096, 5632]))
+    nvec = int(rng.integers(1, 65))
+    def codes(n):
+        b = rng.integers(0, 256, size=n, dtype=np.uint8)
+        if mode == "E5M2":
+            b = np.where((b & 0x7C) == 0x7C, b & 0x83, b).astype(np.uint8)   # no inf / NaN codes
+        return torch.from_numpy(b.view(np.int32).copy()).to(dev).view(torch.uint32)
+    wp, xp = codes(M * K), codes(nvec * K)
+    out = gemv_fp8_batched_acc_fp32_gpu(wp, xp, (M, K), nvec, mode)
+    wd = feather.unpack_fp8_tensor(wp, mode=mode, semantics="kernel").view(M, K).double()
+    xd = feather.unpack_fp8_tensor(xp, mode=mode, semantics="kernel").view(nvec, K).double()
+    want = xd @ wd.T
+    scale = (xd.abs() @ wd.abs().T).max()               # cancellation-free error scale of the fp32 sums
+    assert out.shape == (nvec, M)
+    assert ((out.double() - want).abs().max() / scale).item() <= 1e-5
+
+
 # ---------------------------------------------------------------- dot
 
 def test_dot_docstring_known_answers(dev, kats):

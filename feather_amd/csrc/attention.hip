@@ -169,18 +169,27 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     uint32_t vreg[NU][4];
     auto prefetch = [&](int key0) {
         if (!ALL_STAGE && tid >= UNITS) return;
+        // The tile's first row is wave-uniform (scalar base); the lane adds a 32-bit byte offset inside
+        // the tile, re-derived from the thread index on every call: the index is made opaque here,
+        // otherwise base + offset is hoisted out of the key loop as one 64-bit address per load and
+        // those register pairs are what gets spilled at d = 512 (and a spill reload between two global
+        // loads waits for the first one).
+        const int row0 = __builtin_amdgcn_readfirstlane(key0);
+        const char *kt = reinterpret_cast<const char *>(kh + (int64_t)row0 * DW);
+        const char *vt = reinterpret_cast<const char *>(vh + (int64_t)row0 * DW);
+        int t = tid;
+        asm volatile("" : "+v"(t));
 #pragma unroll
         for (int i = 0; i < NU; i++) {
-            int u = tid + kAttnThreads * i;
-            int key = key0 + u / (D / 16), c16 = u % (D / 16);
+            const int u = t + kAttnThreads * i;
+            const int krel = u / (D / 16), c16 = u % (D / 16);
             kreg[i] = u32x4{0, 0, 0, 0};
-            if (key < L) kreg[i] = *reinterpret_cast<const u32x4 *>(kh + (int64_t)key * DW + 4 * c16);
-            int ddw = u % DW, kg = u / DW;
+            if (key0 + krel < L) kreg[i] = *reinterpret_cast<const u32x4 *>(kt + (uint32_t)(krel * D + 16 * c16));
+            const int ddw = u % DW, kg = u / DW;
+            const uint32_t voff = (uint32_t)(4 * kg * D + 4 * ddw);
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                int vkey = key0 + 4 * kg + r;
-                vreg[i][r] = vkey < L ? vh[(int64_t)vkey * DW + ddw] : 0u;
-            }
+            for (int r = 0; r < 4; r++)
+                vreg[i][r] = key0 + 4 * kg + r < L ? *reinterpret_cast<const uint32_t *>(vt + voff + (uint32_t)(r * D)) : 0u;
         }
     };
     auto stage = [&](int buf) {
@@ -229,6 +238,9 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                 *reinterpret_cast<u32x2 *>(vt_lds + row * VS + (((pos >> 3) ^ swz(row)) << 3) + (pos & 4)) =
                     u32x2{lo2[c], hi2[c]};
             }
+            // d = 512 has no register to spare: keep the scheduler from interleaving the decode of two
+            // units (a spill reload waits for every global load in flight, the tile prefetch included)
+            if constexpr (D >= 512) __builtin_amdgcn_sched_barrier(0);
         }
     };
 

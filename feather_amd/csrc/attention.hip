@@ -238,9 +238,6 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                 *reinterpret_cast<u32x2 *>(vt_lds + row * VS + (((pos >> 3) ^ swz(row)) << 3) + (pos & 4)) =
                     u32x2{lo2[c], hi2[c]};
             }
-            // d = 512 has no register to spare: keep the scheduler from interleaving the decode of two
-            // units (a spill reload waits for every global load in flight, the tile prefetch included)
-            if constexpr (D >= 512) __builtin_amdgcn_sched_barrier(0);
         }
     };
 

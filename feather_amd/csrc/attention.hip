@@ -456,8 +456,8 @@ static int launch_attn(const AttnArgs &a, hipStream_t s) {
 // Workgroup shapes.  A wave of the d = 64 kernel owns 64 queries.  Staging a K/V tile into LDS is
 // shared by the workgroup's waves, and from d = 128 on it is a large share of the vector work, so
 // eight waves (twice the queries per staged tile, two waves per SIMD from one workgroup to overlap
-// the barrier-separated phases) are faster wherever the coarser grid still covers the chip's 256 CUs; d = 256 takes eight waves and 64-key tiles at every
-// length (four independent score chains per wave instead of two).
+// the barrier-separated phases) are faster wherever the coarser grid still covers the chip's 256 CUs;
+// d = 256 takes eight waves at every length.
 template <int MODE, bool VC>
 static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
     const int64_t rows = VC ? a.max_seqlen : a.L, seqs = VC ? a.n_seq : 1;
@@ -478,6 +478,9 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
             // waves (L = 1024: 56.7 -> 48.4 us).  The same split does nothing for d = 512, whose short
             // shapes are bound by decoding K and V once per workgroup whatever the number of queries.
             if (!a.causal && !fills_chip(128)) return launch_attn<256, MODE, 1, 1, 64, 1, VC, 8, 2>(a, s);
+            // long sequences: 32 queries per wave halve the LDS reads per query, which bound this head dim
+            // (L = 8192: 792 -> 640 us); needs 256 workgroups of 256 queries to cover the chip
+            if (fills_chip(256)) return launch_attn<256, MODE, 2, 2, 32, 1, VC, 8>(a, s);
             return launch_attn<256, MODE, 1, 1, 64, 1, VC, 8>(a, s);
         case 512:
             if (fills_chip(128)) return launch_attn<512, MODE, 1, 1, 32, 1, VC, 8>(a, s);

@@ -149,6 +149,8 @@ def test_flash_attention_config_sized_property(dev):
     # eight-wave workgroups: d = 128 and d = 512 switch to them once the coarser grid covers 256 CUs
     ("E5M2", 4, 16, 4096, 128, False), ("E4M3", 4, 16, 1024, 128, True), ("E4M3", 1, 8, 4100, 512, True),
     ("E5M2", 1, 8, 4096, 256, False), ("E4M3", 1, 8, 1024, 256, False),
+    # d = 256 with >= 256 workgroups of 256 queries: 32 queries per wave
+    ("E4M3", 2, 16, 2048, 256, False), ("E5M2", 2, 16, 2048, 256, True), ("E4M3", 1, 8, 8192, 256, False),
 ])
 def test_flash_attention_full_size_rows_vs_fp32_math(dev, mode, B, H, L, d, causal):
     """The remaining attention shapes of the benchmark configurations, too big for the scalar oracle:
@@ -295,6 +297,7 @@ def test_paged_attention_config_shape(dev, orc):
     # the eight-wave d = 64 shape (non-causal, >= 256 groups of 512 queries), lengths around its tile
     ("E5M2", 16, 8, 64, [513, 100, 512, 0] * 4, False),
     ("E4M3", 2, 1, 256, [130, 64, 0, 257], False),           # d = 256 with the key tiles split between wave groups
+    ("E4M3", 16, 8, 256, [257, 100] * 8, True),              # d = 256, 32 queries per wave (>= 256 workgroups)
 ])
 def test_varlen_attention_vs_oracle(dev, orc, mode, n_heads, n_kv, d, lens, causal):
     from feather_amd.routines.attention import flash_attention_fp8_varlen_acc_fp32_gpu

@@ -39,6 +39,7 @@ def _qkv(rng, heads, L, d, mode, orc, ints=False):
     ("E4M3", 1, 64, 256), ("E4M3", 1, 96, 512), ("E5M2", 1, 64, 512), ("E5M2", 8, 1024, 64),
     # d = 256 below 256 workgroups: two wave groups split the key tiles (even, odd and ragged tile counts)
     ("E4M3", 2, 200, 256), ("E5M2", 1, 330, 256), ("E4M3", 1, 128, 256),
+    ("E4M3", 2, 100, 512), ("E5M2", 1, 200, 512),            # the same split at d = 512 (32-key tiles)
 ])
 def test_flash_attention_vs_oracle(dev, orc, mode, heads, L, d):
     from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu

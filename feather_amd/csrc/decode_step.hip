@@ -63,6 +63,10 @@ __device__ __forceinline__ float4 load_parts(const float *p, int n_part, int64_t
 }
 
 // h += delta (if given); xq = pack(fp16(h * rsqrt(mean(h^2) + eps) * w)).  One workgroup per row.
+// The kernel is a chain of memory round trips and little else, so every load of a row's first
+// 4096 elements (h, the norm weights and up to eight partial sums per element) is issued before
+// the first value is used, and the second pass works from registers: two round trips (loads,
+// stores) instead of one per 1024 elements and pass.
 template <int MODE>
 __global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__restrict__ h,
                                                                      const float *__restrict__ delta, int n_part,
@@ -75,45 +79,66 @@ __global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__r
     float4 *hr = reinterpret_cast<float4 *>(h + (int64_t)b * hidden);
     const float *dr = delta ? delta + (int64_t)b * hidden : nullptr;
     const float4 *wr = reinterpret_cast<const float4 *>(w);
-    // the first kKeep values of a thread stay in registers between the two passes
-    constexpr int kKeep = 4;
-    float4 keep[kKeep];
+    const int n4 = hidden / 4;
+    constexpr int kKeep = 4, G = 8;
+    float4 x[kKeep], g[kKeep], part[kKeep][G];
+    // ---- all loads (inactive slots read element 0 and are dropped)
+#pragma unroll
+    for (int it = 0; it < kKeep; it++) {
+        const int i = threadIdx.x + it * kDsThreads, ii = i < n4 ? i : 0;
+        x[it] = hr[ii];
+        g[it] = wr[ii];
+        if (dr) {
+#pragma unroll
+            for (int u = 0; u < G; u++)
+                part[it][u] = *reinterpret_cast<const float4 *>(dr + 4 * ii + (int64_t)min(u, n_part - 1) * part_stride);
+        }
+    }
     float ss = 0.f;
 #pragma unroll
     for (int it = 0; it < kKeep; it++) {
         const int i = threadIdx.x + it * kDsThreads;
-        if (i < hidden / 4) {
-            float4 x = hr[i];
+        if (i < n4) {
             if (dr) {
-                float4 d = load_parts(dr + 4 * i, n_part, part_stride);
-                x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
-                hr[i] = x;
+                float4 d = part[it][0];                      // slices are added in index order
+#pragma unroll
+                for (int u = 1; u < G; u++)
+                    if (u < n_part) { d.x += part[it][u].x; d.y += part[it][u].y; d.z += part[it][u].z; d.w += part[it][u].w; }
+                for (int s0 = G; s0 < n_part; s0 += G) {     // more than G slices: further rounds
+                    float4 q[G];
+#pragma unroll
+                    for (int u = 0; u < G; u++)
+                        q[u] = *reinterpret_cast<const float4 *>(dr + 4 * i + (int64_t)min(s0 + u, n_part - 1) * part_stride);
+#pragma unroll
+                    for (int u = 0; u < G; u++)
+                        if (s0 + u < n_part) { d.x += q[u].x; d.y += q[u].y; d.z += q[u].z; d.w += q[u].w; }
+                }
+                x[it].x += d.x; x[it].y += d.y; x[it].z += d.z; x[it].w += d.w;
+                hr[i] = x[it];
             }
-            keep[it] = x;
-            ss += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+            ss += (x[it].x * x[it].x + x[it].y * x[it].y) + (x[it].z * x[it].z + x[it].w * x[it].w);
         }
     }
-    for (int i = threadIdx.x + kKeep * kDsThreads; i < hidden / 4; i += kDsThreads) {
-        float4 x = hr[i];
+    for (int i = threadIdx.x + kKeep * kDsThreads; i < n4; i += kDsThreads) {   // rows longer than 4096
+        float4 y = hr[i];
         if (dr) {
             float4 d = load_parts(dr + 4 * i, n_part, part_stride);
-            x.x += d.x; x.y += d.y; x.z += d.z; x.w += d.w;
-            hr[i] = x;
+            y.x += d.x; y.y += d.y; y.z += d.z; y.w += d.w;
+            hr[i] = y;
         }
-        ss += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+        ss += (y.x * y.x + y.y * y.y) + (y.z * y.z + y.w * y.w);
     }
     const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
 #pragma unroll
     for (int it = 0; it < kKeep; it++) {
         const int i = threadIdx.x + it * kDsThreads;
-        if (i < hidden / 4) {
-            float4 x = keep[it], g = wr[i];
-            xq[(int64_t)b * (hidden / 4) + i] = quant4<MODE>(x.x * r * g.x, x.y * r * g.y, x.z * r * g.z, x.w * r * g.w);
-        }
+        if (i < n4)
+            xq[(int64_t)b * n4 + i] = quant4<MODE>(x[it].x * r * g[it].x, x[it].y * r * g[it].y, x[it].z * r * g[it].z,
+                                                  x[it].w * r * g[it].w);
     }
-    for (int i = threadIdx.x + kKeep * kDsThreads; i < hidden / 4; i += kDsThreads) {
-        float4 x = hr[i], g = wr[i];
-        xq[(int64_t)b * (hidden / 4) + i] = quant4<MODE>(x.x * r * g.x, x.y * r * g.y, x.z * r * g.z, x.w * r * g.w);
+    for (int i = threadIdx.x + kKeep * kDsThreads; i < n4; i += kDsThreads) {
+        float4 y = hr[i], gg = wr[i];
+        xq[(int64_t)b * n4 + i] = quant4<MODE>(y.x * r * gg.x, y.y * r * gg.y, y.z * r * gg.z, y.w * r * gg.w);
     }
 }
 
@@ -154,13 +179,43 @@ __global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *
     const int item = blockIdx.y * kRopeThreads + threadIdx.x;
     const bool live = item < heads * half_w;
     const int head = live ? item / half_w : 0, t = live ? item % half_w : 0;
-    // the GEMV partials do not depend on the position: their loads go out before the lookups below
+    // Two chains of loads: position -> block id, and the GEMV partials of the two elements this
+    // thread rotates.  The position goes out first, then every partial (up to 8 slices per element),
+    // then the block id as soon as the position is back: the chains overlap instead of queueing.
+    const int pos_raw = ctx_lens[b];
     const float *x = qkv + ((int64_t)b * heads + head) * d;
-    float4 lo = load_parts(x + 4 * t, n_part, part_stride);          // elements 4t .. 4t+3
-    float4 hi = load_parts(x + d / 2 + 4 * t, n_part, part_stride);  // their partners
-    const int pos = min(ctx_lens[b], max_blocks * block_size - 1);
+    constexpr int G = 8;
+    float4 pl[G], ph[G];
+#pragma unroll
+    for (int u = 0; u < G; u++) {
+        const int64_t off = (int64_t)min(u, n_part - 1) * part_stride;
+        pl[u] = *reinterpret_cast<const float4 *>(x + 4 * t + off);            // elements 4t .. 4t+3
+        ph[u] = *reinterpret_cast<const float4 *>(x + d / 2 + 4 * t + off);    // their partners
+    }
+    const int pos = min(pos_raw, max_blocks * block_size - 1);
     if (threadIdx.x == 0 && blockIdx.y == 0) ctx_after[b] = pos + 1;
     const int64_t slot = ((int64_t)block_tables[(int64_t)b * max_blocks + pos / block_size] * n_kv) * block_size;
+    float4 lo = pl[0], hi = ph[0];                   // slices are added in index order
+#pragma unroll
+    for (int u = 1; u < G; u++)
+        if (u < n_part) {
+            lo.x += pl[u].x; lo.y += pl[u].y; lo.z += pl[u].z; lo.w += pl[u].w;
+            hi.x += ph[u].x; hi.y += ph[u].y; hi.z += ph[u].z; hi.w += ph[u].w;
+        }
+    for (int s0 = G; s0 < n_part; s0 += G) {          // more than G slices: further rounds
+#pragma unroll
+        for (int u = 0; u < G; u++) {
+            const int64_t off = (int64_t)min(s0 + u, n_part - 1) * part_stride;
+            pl[u] = *reinterpret_cast<const float4 *>(x + 4 * t + off);
+            ph[u] = *reinterpret_cast<const float4 *>(x + d / 2 + 4 * t + off);
+        }
+#pragma unroll
+        for (int u = 0; u < G; u++)
+            if (s0 + u < n_part) {
+                lo.x += pl[u].x; lo.y += pl[u].y; lo.z += pl[u].z; lo.w += pl[u].w;
+                hi.x += ph[u].x; hi.y += ph[u].y; hi.z += ph[u].z; hi.w += ph[u].w;
+            }
+    }
     if (!live) return;
     {
         if (head < n_q + n_kv) {

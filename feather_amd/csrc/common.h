@@ -221,16 +221,18 @@ __device__ __forceinline__ float wave_sum(float x) {
 // second, v_permlane32_swap the upper half of the first with the lower half of the second; with
 // both operands holding x, every lane then finds x and its partner's x in the two registers.
 // (Inline assembly: the compiler folds the two results of the corresponding builtins into one when
-// both inputs are the same value.  s_nop 1 covers the VALU-write -> permlane-read wait states.)
+// both inputs are the same value.  The copy and the final v_max_f32 are part of the statement so that
+// exactly one copy is made and the compiler adds no canonicalising max(x, x) on values it cannot see
+// through; s_nop 1 covers the VALU-write -> permlane-read wait states.)
 __device__ __forceinline__ float max_xor16(float x) {
-    float a = x, b = x;
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
-    return fmaxf(a, b);
+    float a = x, b;
+    asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_max_f32 %0, %0, %1" : "+v"(a), "=&v"(b));
+    return a;
 }
 __device__ __forceinline__ float max_xor32(float x) {
-    float a = x, b = x;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
-    return fmaxf(a, b);
+    float a = x, b;
+    asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_max_f32 %0, %0, %1" : "+v"(a), "=&v"(b));
+    return a;
 }
 
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }

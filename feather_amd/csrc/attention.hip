@@ -1,12 +1,13 @@
 // Flash-attention forward on FP8-packed Q/K/V (prefill): fixed-length heads, or variable-length
 // sequences packed back to back with an optional causal mask.
 //
-// Work split.  One workgroup (WAVES waves, 4 or 8) owns a tile of 16*QB*WAVES
-// queries of one head; each wave owns 16*QB of them for the whole key loop.  Keys/values are
+// Work split.  One workgroup (WAVES waves, 4 or 8) owns a tile of 16*QB*WAVES/KSPLIT
+// queries of one head; each wave owns 16*QB of them for the whole key loop (with KSPLIT = 2 two
+// waves share them and alternate over the key tiles).  Keys/values are
 // streamed in tiles of BN keys: the PACKED tile is fetched from global memory
-// into registers one tile ahead (so HBM/L2 latency overlaps the MFMA work of
-// the current tile), decoded to fp16 on its way into LDS, and read from LDS as
-// MFMA operands by every wave.
+// into registers two tiles ahead (so HBM/L2 latency overlaps the MFMA work of
+// the tiles before it), decoded to fp16 on its way into the other LDS buffer one tile
+// ahead, and read from LDS as MFMA operands by every wave.
 //
 // Matrix cores.  Everything is computed transposed so that one lane keeps one
 // query for the whole kernel:

@@ -25,7 +25,14 @@
 // the lane's dot product sits on the diagonal of its 4x4 block) is exact and
 // changes nothing: E4M3 45.2 us either way.  (4) Plain instead of non-temporal
 // loads: 48.8 us.  Buffer loads (any cache policy) instead of global loads: no
-// gain once the row bases are wave-uniform.
+// gain once the row bases are wave-uniform.  (5) E4M3 through the hardware's
+// FP8 -> fp16 conversion (v_cvt_scalef32_pk_f16_fp8: 9 instructions per word
+// with the check below instead of 14) with the exact decode as a wave-uniform
+// fallback for batches that hold a code on which the two differ (zero exponent
+// with a non-zero mantissa: OCP subnormals against the reference's raw mantissa
+// bits; 0x7F / 0xFF).  Correct, but the RNE packer emits those subnormal codes
+// for every |x| < 2^-6, 1-2 % of N(0,1) data, so every batch of a wave (8192
+// codes) falls back and pays for both decodes: 64 us.
 //
 // A workgroup takes a contiguous range of rows so the vector decode is
 // amortised; ranges are sized so that the grid is a few workgroups per CU.

@@ -250,7 +250,7 @@ def main() -> int:
             cl = torch.randint(512, cmax, (batch,), generator=g, device=dev, dtype=torch.int32)
             tok = torch.randint(0, cfg.vocab, (batch,), generator=g, device=dev, dtype=torch.int32)
             logits = torch.empty((batch, cfg.vocab), dtype=torch.float32, device=dev)
-            us = gpu_time_us(lambda i: dec.step(tok, btd, cl, out=logits), 20, 3, sync)
+            us = gpu_time_us(lambda i: dec.step(tok, btd, cl, out=logits), 20, 10, sync)
             step_bytes = dec.weight_bytes() + int(cl.sum().item()) * 2 * cfg.n_kv_heads * cfg.head_dim * cfg.n_layers
             key = f"decode_tinyllama_b{batch}_{mode.lower()}"
             extra[key + "_ms_per_step"] = round(us / 1e3, 3)

@@ -266,6 +266,12 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         if (!skip) {
 
         half8_t pf[QB][KB32];
+        // PVB: with several query blocks per wave and a V^T tile small enough to sit in registers
+        // (d = 64: 8 fragments), every block's P.V MFMAs follow its softmax directly, so they run on
+        // the matrix core while the vector ALU works through the next block's exponentials; otherwise
+        // all blocks share each V^T fragment as it is read from LDS, after the last softmax
+        constexpr bool PVB = BF8 && QB > 1 && DB * KB32 <= 8;   // (the fp16 score path has no registers left for it)
+        half8_t vres[PVB ? KB32 : 1][PVB ? DB : 1];
         // query blocks are scored SB at a time: the K fragments are re-used across the SB
         // blocks while only SB * KB16 score tiles are live in registers
 #pragma unroll
@@ -289,6 +295,16 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                         for (int b = 0; b < SB; b++)
                             s[b][c] = mfma16(kf, qf[b0 + b][st], st == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : s[b][c]);
                     }
+                }
+            }
+            if constexpr (PVB) {
+                if (b0 == 0) {
+#pragma unroll
+                    for (int t = 0; t < KB32; t++)
+#pragma unroll
+                        for (int d = 0; d < DB; d++)
+                            vres[t][d] = *reinterpret_cast<const half8_t *>(vt_lds + (16 * d + j) * VS +
+                                                                            (((4 * t + kb) ^ swz(16 * d + j)) << 3));
                 }
             }
             // ---- online softmax, one query per lane column.  The running maximum is kept on
@@ -336,10 +352,19 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
 #pragma unroll
                     for (int d = 0; d <= DB; d++) o[b0 + b][d] *= alpha;
                 }
+                if constexpr (PVB) {
+#pragma unroll
+                    for (int t = 0; t < KB32; t++) {
+#pragma unroll
+                        for (int d = 0; d < DB; d++) o[b0 + b][d] = mfma16(vres[t][d], pf[b0 + b][t], o[b0 + b][d]);
+                        o[b0 + b][DB] = mfma16(ones, pf[b0 + b][t], o[b0 + b][DB]);
+                    }
+                }
             }
         }
 
         // ---- O^T += V^T P^T (and the row sums through the constant ones block)
+        if constexpr (!PVB)
 #pragma unroll
         for (int t = 0; t < KB32; t++) {
 #pragma unroll

@@ -265,13 +265,100 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         if constexpr (KSPLIT > 1) skip = skip || (key0 / BN) % KSPLIT != kgroup;   // another group's tile
         if (!skip) {
 
+        // ---- online softmax of one 16-query block, one query per lane column.  The running maximum
+        // is kept on the raw scores; scale * log2(e) is folded into one fma per score:
+        // p = 2^(s * c - m * c).  Leaves P (fp16) in pb and rescales the block's accumulators if needed.
+        auto softmax_block = [&](int qb, float4_t (&sb)[KB16], half8_t (&pb)[KB32]) {
+            if (ragged || diag) {
+                int last = diag ? min(L - 1, q0 + 16 * qb + j) : L - 1;   // last visible key
+                // opaque to the optimiser from here on: otherwise the 16 key-index compares below
+                // are hoisted out of this rarely taken branch and run for every tile
+                asm volatile("" : "+v"(last));
+                const int rel = last - key0 - 4 * kb;   // key 16 c + 4 kb + r of the tile is hidden if 16 c + r > rel
+#pragma unroll
+                for (int c = 0; c < KB16; c++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (16 * c + r > rel) sb[c][r] = -INFINITY;
+            }
+            float mx = sb[0][0];
+#pragma unroll
+            for (int c = 0; c < KB16; c++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) mx = fmaxf(mx, sb[c][r]);
+            mx = max_xor32(max_xor16(mx));   // over the four lanes that share the query
+            const float m_old = m_run[qb];
+            const float m_new = fmaxf(m_old, mx);
+            const float mc = m_new * scale_log2e;
+#pragma unroll
+            for (int t = 0; t < KB32; t++) {
+                half8_t p8;
+#pragma unroll
+                for (int a = 0; a < 2; a++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sb[2 * t + a][r], scale_log2e, -mc));
+                        p8[4 * a + r] = (_Float16)e;  // round to nearest even, as P.to(fp16)
+                    }
+                pb[t] = p8;
+            }
+            // rescale only when some query of this block saw a new maximum (wave-uniform test)
+            if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
+                const float alpha = __builtin_amdgcn_exp2f((m_old - m_new) * scale_log2e);
+                m_run[qb] = m_new;
+#pragma unroll
+                for (int d = 0; d <= DB; d++) o[qb][d] *= alpha;
+            }
+        };
+        // PVB: with several query blocks per wave, one-byte (bf8) K fragments and K / V^T tiles small
+        // enough to sit in registers (d = 64: 8 + 8 fragments), the blocks go through score -> softmax ->
+        // P.V one after the other with the scores one block ahead: the MFMAs of block b's P.V and of
+        // block b + 2's scores run on the matrix core while the vector ALU works through block b + 1's
+        // exponentials (d = 64, L = 8192: 1189 -> 1147 us).  The fp16 score path has no registers left
+        // for resident K fragments (spills) and re-reading them from LDS per block costs more than the
+        // overlap gains (1250 -> 1262 / 1275 us), so there, and for the wider heads, all blocks share
+        // each K / V^T fragment as it is read from LDS.
+        constexpr bool PVB = BF8 && QB > 1 && DB * KB32 <= 8 && KB16 * STEPS <= 8;
+        if constexpr (PVB) {
+            long kres[KB16][STEPS];
+            half8_t vres[KB32][DB];
+#pragma unroll
+            for (int c = 0; c < KB16; c++)
+#pragma unroll
+                for (int st = 0; st < STEPS; st++)
+                    kres[c][st] = *reinterpret_cast<const long *>(reinterpret_cast<const unsigned char *>(k_lds) +
+                                                                  (16 * c + j) * (2 * KS) + 32 * st + 8 * kb);
+#pragma unroll
+            for (int t = 0; t < KB32; t++)
+#pragma unroll
+                for (int d = 0; d < DB; d++)
+                    vres[t][d] = *reinterpret_cast<const half8_t *>(vt_lds + (16 * d + j) * VS +
+                                                                    (((4 * t + kb) ^ swz(16 * d + j)) << 3));
+            float4_t s2[2][KB16];
+            auto score = [&](int qb, float4_t (&sb)[KB16]) {
+#pragma unroll
+                for (int c = 0; c < KB16; c++)
+#pragma unroll
+                    for (int st = 0; st < STEPS; st++) {
+                        const float4_t acc0 = st == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : sb[c];
+                        sb[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(kres[c][st], qf8[qb][st], acc0, 0, 0, 0);
+                    }
+            };
+            score(0, s2[0]);
+#pragma unroll
+            for (int b = 0; b < QB; b++) {
+                if (b + 1 < QB) score(b + 1, s2[(b + 1) & 1]);
+                half8_t pb[KB32];
+                softmax_block(b, s2[b & 1], pb);
+#pragma unroll
+                for (int t = 0; t < KB32; t++) {
+#pragma unroll
+                    for (int d = 0; d < DB; d++) o[b][d] = mfma16(vres[t][d], pb[t], o[b][d]);
+                    o[b][DB] = mfma16(ones, pb[t], o[b][DB]);
+                }
+            }
+        } else {
         half8_t pf[QB][KB32];
-        // PVB: with several query blocks per wave and a V^T tile small enough to sit in registers
-        // (d = 64: 8 fragments), every block's P.V MFMAs follow its softmax directly, so they run on
-        // the matrix core while the vector ALU works through the next block's exponentials; otherwise
-        // all blocks share each V^T fragment as it is read from LDS, after the last softmax
-        constexpr bool PVB = BF8 && QB > 1 && DB * KB32 <= 8;   // (the fp16 score path has no registers left for it)
-        half8_t vres[PVB ? KB32 : 1][PVB ? DB : 1];
         // query blocks are scored SB at a time: the K fragments are re-used across the SB
         // blocks while only SB * KB16 score tiles are live in registers
 #pragma unroll
@@ -297,74 +384,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                     }
                 }
             }
-            if constexpr (PVB) {
-                if (b0 == 0) {
 #pragma unroll
-                    for (int t = 0; t < KB32; t++)
-#pragma unroll
-                        for (int d = 0; d < DB; d++)
-                            vres[t][d] = *reinterpret_cast<const half8_t *>(vt_lds + (16 * d + j) * VS +
-                                                                            (((4 * t + kb) ^ swz(16 * d + j)) << 3));
-                }
-            }
-            // ---- online softmax, one query per lane column.  The running maximum is kept on
-            // the raw scores; scale * log2(e) is folded into one fma per score:
-            // p = 2^(s * c - m * c).
-#pragma unroll
-            for (int b = 0; b < SB; b++) {
-                if (ragged || diag) {
-                    int last = diag ? min(L - 1, q0 + 16 * (b0 + b) + j) : L - 1;   // last visible key
-                    // opaque to the optimiser from here on: otherwise the 16 key-index compares below
-                    // are hoisted out of this rarely taken branch and run for every tile
-                    asm volatile("" : "+v"(last));
-                    const int rel = last - key0 - 4 * kb;   // key 16 c + 4 kb + r of the tile is hidden if 16 c + r > rel
-#pragma unroll
-                    for (int c = 0; c < KB16; c++)
-#pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            if (16 * c + r > rel) s[b][c][r] = -INFINITY;
-                }
-                float mx = s[b][0][0];
-#pragma unroll
-                for (int c = 0; c < KB16; c++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++) mx = fmaxf(mx, s[b][c][r]);
-                mx = max_xor32(max_xor16(mx));   // over the four lanes that share the query
-                const float m_old = m_run[b0 + b];
-                const float m_new = fmaxf(m_old, mx);
-                const float mc = m_new * scale_log2e;
-#pragma unroll
-                for (int t = 0; t < KB32; t++) {
-                    half8_t p8;
-#pragma unroll
-                    for (int a = 0; a < 2; a++)
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[b][2 * t + a][r], scale_log2e, -mc));
-                            p8[4 * a + r] = (_Float16)e;  // round to nearest even, as P.to(fp16)
-                        }
-                    pf[b0 + b][t] = p8;
-                }
-                // rescale only when some query of this block saw a new maximum (wave-uniform test)
-                if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
-                    const float alpha = __builtin_amdgcn_exp2f((m_old - m_new) * scale_log2e);
-                    m_run[b0 + b] = m_new;
-#pragma unroll
-                    for (int d = 0; d <= DB; d++) o[b0 + b][d] *= alpha;
-                }
-                if constexpr (PVB) {
-#pragma unroll
-                    for (int t = 0; t < KB32; t++) {
-#pragma unroll
-                        for (int d = 0; d < DB; d++) o[b0 + b][d] = mfma16(vres[t][d], pf[b0 + b][t], o[b0 + b][d]);
-                        o[b0 + b][DB] = mfma16(ones, pf[b0 + b][t], o[b0 + b][DB]);
-                    }
-                }
-            }
+            for (int b = 0; b < SB; b++) softmax_block(b0 + b, s[b], pf[b0 + b]);
         }
 
         // ---- O^T += V^T P^T (and the row sums through the constant ones block)
-        if constexpr (!PVB)
 #pragma unroll
         for (int t = 0; t < KB32; t++) {
 #pragma unroll
@@ -377,6 +401,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
 #pragma unroll
             for (int b = 0; b < QB; b++) o[b][DB] = mfma16(ones, pf[b][t], o[b][DB]);
         }
+        }   // !PVB
         }   // !skip
         __syncthreads();  // tile i+1 is visible; every wave is done reading tile i
     }

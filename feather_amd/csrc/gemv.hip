@@ -32,7 +32,20 @@
 // with a non-zero mantissa: OCP subnormals against the reference's raw mantissa
 // bits; 0x7F / 0xFF).  Correct, but the RNE packer emits those subnormal codes
 // for every |x| < 2^-6, 1-2 % of N(0,1) data, so every batch of a wave (8192
-// codes) falls back and pays for both decodes: 64 us.
+// codes) falls back and pays for both decodes: 64 us.  (6) Per-wave time
+// stamps (s_memrealtime) show that the two waves of a SIMD do not advance
+// together: the older one wins the vector ALU whenever both have data and ends
+// 6-11 us before the younger one in E4M3 mode (3 us in E5M2), all workgroups
+// ending within 3 us of each other.  Levelling the two through s_setprio (each
+// wave publishes its step count in LDS, the one behind raises its priority)
+// shrinks that spread to 3 us and leaves the time where it was (43.5 -> 42.8-44.1
+// us): the memory system is as busy with four waves per CU in the last
+// microseconds as with eight.  (7) Fetching the vector with 128-bit loads and the
+// first group of matrix loads before the vector is decoded into LDS (the kernel
+// otherwise starts with two dependent memory latencies, ~2 us): -0.5 us for E5M2
+// at 16384^2 (-1.0 us on uniform random codes), +0.4 us for E4M3 and for both
+// modes at 8192^2; with the matrix loads issued first the vector words queue
+// behind them (+2.4 us).
 //
 // A workgroup takes a contiguous range of rows so the vector decode is
 // amortised; ranges are sized so that the grid is a few workgroups per CU.

@@ -264,6 +264,44 @@ def test_paged_attention_split_bookkeeping(dev, orc, mode, n_seq, Hq, Hkv, d, bs
     assert not out[ctx == 0].any()
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_paged_attention_random_shapes(dev, orc, seed):
+    """Random head groupings, head dims, block sizes (powers of two and not), context bounds around the
+    512-token split and contexts from empty to the bound, against the oracle."""
+    from feather_amd.routines.paged_attention import paged_attention_fp8_acc_fp32_gpu
+    rng = np.random.default_rng(1000 + seed)
+    mode = ("E5M2", "E4M3")[seed % 2]
+    d = int(rng.choice([64, 64, 128, 256]))
+    group = int(rng.choice([1, 2, 3, 4, 8, 16]))
+    Hkv = int(rng.integers(1, 4))
+    Hq = group * Hkv
+    bs = int(rng.choice([4, 8, 16, 32, 5, 12, 24]))
+    max_ctx = int(rng.choice([1, 31, 200, 512, 513, 1024, 1025, 1400]))
+    n_seq = int(rng.integers(1, 7))
+    max_blocks = (max_ctx + bs - 1) // bs
+    n_blocks = n_seq * max_blocks + 2
+    ctx = rng.integers(0, max_ctx + 1, size=n_seq).astype(np.int32)
+    ctx[rng.integers(0, n_seq)] = max_ctx
+    kc = orc.pack_fp8(rng.standard_normal((n_blocks, Hkv, bs, d)).astype(np.float16), mode).reshape(n_blocks, -1)
+    vc = orc.pack_fp8(rng.standard_normal((n_blocks, Hkv, bs, d)).astype(np.float16), mode).reshape(n_blocks, -1)
+    poison = n_blocks - 1
+    kc[poison] = vc[poison] = 0x7F7F7F7F
+    q = orc.pack_fp8((2.0 * rng.standard_normal((n_seq, Hq, d))).astype(np.float16), mode)
+    bt = rng.permutation(n_blocks - 1)[: n_seq * max_blocks].reshape(n_seq, max_blocks).astype(np.int32)
+    for i in range(n_seq):
+        bt[i, (ctx[i] + bs - 1) // bs:] = poison
+    print(f"seed {seed}: {mode} n_seq {n_seq} Hq {Hq} Hkv {Hkv} d {d} bs {bs} max_ctx {max_ctx} ctx {ctx.tolist()}", flush=True)
+    out = paged_attention_fp8_acc_fp32_gpu(
+        _dev_words(q, dev, (n_seq, Hq, d // 4)), _dev_words(kc, dev, (n_blocks, Hkv, bs, d // 4)),
+        _dev_words(vc, dev, (n_blocks, Hkv, bs, d // 4)), torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev),
+        mode=mode, max_context_len=max_ctx).cpu().numpy()
+    live = np.flatnonzero(ctx > 0)
+    want = orc.paged_attn(q.reshape(n_seq, -1)[live], kc, vc, bt[live], ctx[live], Hq, Hkv, d, bs, mode)
+    assert np.isfinite(want).all()
+    assert _nerr(out[live], want) <= TOL
+    assert not out[ctx == 0].any()
+
+
 def test_paged_attention_config_shape(dev, orc):
     """TinyLlama-shaped decode attention: batch 32, 32 query / 4 KV heads, d 64, block 16,
     contexts uniform in [512, 4096], permuted block table."""

@@ -3,7 +3,7 @@
 //
 // Work split.  One workgroup (WAVES waves, 4 or 8) owns a tile of 16*QB*WAVES/KSPLIT
 // queries of one head; each wave owns 16*QB of them for the whole key loop (with KSPLIT = 2 two
-// waves share them and alternate over the key tiles).  Keys/values are
+// waves share them and each scores one half of the keys of every tile).  Keys/values are
 // streamed in tiles of BN keys: the PACKED tile is fetched from global memory
 // into registers two tiles ahead (so HBM/L2 latency overlaps the MFMA work of
 // the tiles before it), decoded to fp16 on its way into the other LDS buffer one tile
@@ -34,6 +34,7 @@
 // rounded to fp16 before P.V, fp32 output.  One difference inside the stated
 // tolerance: the denominator sums the fp16-rounded P (the values that multiply
 // V) where the reference sums P before rounding.
+#include <type_traits>
 #include "common.h"
 
 namespace feather {
@@ -63,10 +64,13 @@ __device__ __forceinline__ half8_t dec8(uint32_t w0, uint32_t w1) {
 //     cu_seqlens (n_seq + 1 row offsets) occupies rows [cu[s], cu[s+1]) of every head and
 //     attends only to itself; with causal != 0 query i sees keys 0..i of its sequence.
 //     tiles_per_head = n_seq * tiles_per_seq; L, keys_scored and mask_tail are not used.
-// KSPLIT  wave groups that share the workgroup's queries and take the key tiles round robin
-//         (tile t goes to group t % KSPLIT), merged through LDS at the end: finer work items for
-//         grids that would leave CUs idle.  Group 0 always has tile 0, so its running maximum is
-//         finite whenever the sequence has a key; not combined with the causal mask.
+// KSPLIT  wave groups that share the workgroup's queries: group g scores keys [g, g + 1) * BN / KSPLIT of
+//         every tile with its own running maximum, sum and accumulators, merged through LDS at the
+//         end (finer work items for grids that would leave CUs idle; every wave is busy in every
+//         tile, where groups that took whole tiles in turn idled at the tile barrier while the other
+//         one worked).  A group of 16 keys multiplies P and V on the 16x16x16 MFMA.  Group 0 always has
+//         key 0, so its running maximum is finite whenever the sequence has a key; not combined with
+//         the causal mask.
 template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC, int WAVES = 4, int KSPLIT = 1>
 __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     const uint32_t *__restrict__ q, const uint32_t *__restrict__ k, const uint32_t *__restrict__ v,
@@ -91,6 +95,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     constexpr bool ALL_STAGE = UNITS >= kAttnThreads;
     static_assert(UNITS % 64 == 0 && (ALL_STAGE ? UNITS % kAttnThreads == 0 : true), "tile / workgroup mismatch");
     constexpr int KB16 = BN / 16, KB32 = BN / 32, DB = D / 16, STEPS = D / 32;
+    constexpr int GBN = BN / KSPLIT;       // keys of a tile that one key group scores
+    static_assert(GBN == 16 || GBN % 32 == 0, "a key group scores 16 keys or whole groups of 32");
+    constexpr bool K16 = GBN == 16;
+    constexpr int GKB16 = GBN / 16, GKB32 = K16 ? 1 : GBN / 32;
+    using pfrag_t = std::conditional_t<K16, half4_t, half8_t>;   // P of one 16- or 32-key MFMA step
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     // two buffers of (K tile, V^T tile): tile i+1 is written while tile i is being read
@@ -250,7 +259,12 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     for (int key0 = 0; key0 < keys_scored; key0 += BN, cur ^= 1) {
         // tile i+1 goes to the other buffer (its readers passed the barrier that ended the previous
         // iteration) and tile i+2 into registers, both off the critical path of this tile's math
-        if (key0 + BN < keys_scored) {
+        // At d = 512 the two waves that share a SIMD (w and w + 4 of an eight-wave workgroup) run this
+        // in opposite order, math first for the second one: staging is vector-ALU work, the math is LDS
+        // reads and MFMAs, and in lock step the pair wants the same unit at the same time (-2..5 % time;
+        // the narrower heads lose 1-4 % with it, their staging is a smaller share of a tile).
+        const bool math_first = WAVES == 8 && D >= 512 && wave >= 4;
+        if (!math_first && key0 + BN < keys_scored) {
             stage(cur ^ 1);
             if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
         }
@@ -262,45 +276,54 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
             diag = causal && key0 + BN - 1 > q0;          // some key of the tile lies past the wave's first query
             skip = causal && key0 > q0 + 16 * QB - 1;     // every key lies past the wave's last query
         }
-        if constexpr (KSPLIT > 1) skip = skip || (key0 / BN) % KSPLIT != kgroup;   // another group's tile
+        if constexpr (KSPLIT > 1) skip = skip || (mask_tail && key0 + kgroup * GBN >= L);   // no key of this group's part exists
         if (!skip) {
 
         // ---- online softmax of one 16-query block, one query per lane column.  The running maximum
         // is kept on the raw scores; scale * log2(e) is folded into one fma per score:
         // p = 2^(s * c - m * c).  Leaves P (fp16) in pb and rescales the block's accumulators if needed.
-        auto softmax_block = [&](int qb, float4_t (&sb)[KB16], half8_t (&pb)[KB32]) {
+        auto softmax_block = [&](int qb, float4_t (&sb)[GKB16], pfrag_t (&pb)[GKB32]) {
             if (ragged || diag) {
                 int last = diag ? min(L - 1, q0 + 16 * qb + j) : L - 1;   // last visible key
                 // opaque to the optimiser from here on: otherwise the 16 key-index compares below
                 // are hoisted out of this rarely taken branch and run for every tile
                 asm volatile("" : "+v"(last));
-                const int rel = last - key0 - 4 * kb;   // key 16 c + 4 kb + r of the tile is hidden if 16 c + r > rel
+                // key 16 c + 4 kb + r of the group's part of the tile is hidden if 16 c + r > rel
+                const int rel = last - key0 - kgroup * GBN - 4 * kb;
 #pragma unroll
-                for (int c = 0; c < KB16; c++)
+                for (int c = 0; c < GKB16; c++)
 #pragma unroll
                     for (int r = 0; r < 4; r++)
                         if (16 * c + r > rel) sb[c][r] = -INFINITY;
             }
             float mx = sb[0][0];
 #pragma unroll
-            for (int c = 0; c < KB16; c++)
+            for (int c = 0; c < GKB16; c++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) mx = fmaxf(mx, sb[c][r]);
             mx = max_xor32(max_xor16(mx));   // over the four lanes that share the query
             const float m_old = m_run[qb];
             const float m_new = fmaxf(m_old, mx);
             const float mc = m_new * scale_log2e;
+            if constexpr (K16) {
+                half4_t p4;
 #pragma unroll
-            for (int t = 0; t < KB32; t++) {
-                half8_t p8;
+                for (int r = 0; r < 4; r++)
+                    p4[r] = (_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(sb[0][r], scale_log2e, -mc));
+                pb[0] = p4;
+            } else {
 #pragma unroll
-                for (int a = 0; a < 2; a++)
+                for (int t = 0; t < GKB32; t++) {
+                    half8_t p8;
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sb[2 * t + a][r], scale_log2e, -mc));
-                        p8[4 * a + r] = (_Float16)e;  // round to nearest even, as P.to(fp16)
-                    }
-                pb[t] = p8;
+                    for (int a = 0; a < 2; a++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sb[2 * t + a][r], scale_log2e, -mc));
+                            p8[4 * a + r] = (_Float16)e;  // round to nearest even, as P.to(fp16)
+                        }
+                    pb[t] = p8;
+                }
             }
             // rescale only when some query of this block saw a new maximum (wave-uniform test)
             if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
@@ -318,7 +341,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         // for resident K fragments (spills) and re-reading them from LDS per block costs more than the
         // overlap gains (1250 -> 1262 / 1275 us), so there, and for the wider heads, all blocks share
         // each K / V^T fragment as it is read from LDS.
-        constexpr bool PVB = BF8 && QB > 1 && DB * KB32 <= 8 && KB16 * STEPS <= 8;
+        constexpr bool PVB = KSPLIT == 1 && BF8 && QB > 1 && DB * KB32 <= 8 && KB16 * STEPS <= 8;
         if constexpr (PVB) {
             long kres[KB16][STEPS];
             half8_t vres[KB32][DB];
@@ -358,26 +381,27 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                 }
             }
         } else {
-        half8_t pf[QB][KB32];
+        pfrag_t pf[QB][GKB32];
+        const int kc0 = kgroup * GKB16;   // first 16-key block of this key group inside the tile
         // query blocks are scored SB at a time: the K fragments are re-used across the SB
-        // blocks while only SB * KB16 score tiles are live in registers
+        // blocks while only SB * GKB16 score tiles are live in registers
 #pragma unroll
         for (int b0 = 0; b0 < QB; b0 += SB) {
             // ---- S^T = K Q^T (raw, unscaled scores)
-            float4_t s[SB][KB16];
+            float4_t s[SB][GKB16];
 #pragma unroll
-            for (int c = 0; c < KB16; c++) {
+            for (int c = 0; c < GKB16; c++) {
 #pragma unroll
                 for (int st = 0; st < STEPS; st++) {
                     if constexpr (BF8) {
                         const long kf = *reinterpret_cast<const long *>(reinterpret_cast<const unsigned char *>(k_lds) +
-                                                                       (16 * c + j) * (2 * KS) + 32 * st + 8 * kb);
+                                                                       (16 * (kc0 + c) + j) * (2 * KS) + 32 * st + 8 * kb);
 #pragma unroll
                         for (int b = 0; b < SB; b++)
                             s[b][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(
                                 kf, qf8[b0 + b][st], st == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : s[b][c], 0, 0, 0);
                     } else {
-                        half8_t kf = *reinterpret_cast<const half8_t *>(k_lds + (16 * c + j) * KS + 32 * st + 8 * kb);
+                        half8_t kf = *reinterpret_cast<const half8_t *>(k_lds + (16 * (kc0 + c) + j) * KS + 32 * st + 8 * kb);
 #pragma unroll
                         for (int b = 0; b < SB; b++)
                             s[b][c] = mfma16(kf, qf[b0 + b][st], st == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : s[b][c]);
@@ -389,27 +413,47 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         }
 
         // ---- O^T += V^T P^T (and the row sums through the constant ones block)
+        if constexpr (K16) {
+            // keys 16 a + 4 kb + r of 32-key group t sit at slots 8 kb + 4 a + r of a V^T row: the four
+            // keys of this lane are half a chunk
+            const int t = kgroup / 2, a = kgroup % 2;
+            const half4_t ones4 = {one_or_zero, one_or_zero, one_or_zero, one_or_zero};
 #pragma unroll
-        for (int t = 0; t < KB32; t++) {
+            for (int d = 0; d < DB; d++) {
+                half4_t vf = *reinterpret_cast<const half4_t *>(vt_lds + (16 * d + j) * VS +
+                                                                (((4 * t + kb) ^ swz(16 * d + j)) << 3) + 4 * a);
+#pragma unroll
+                for (int b = 0; b < QB; b++) o[b][d] = __builtin_amdgcn_mfma_f32_16x16x16f16(vf, pf[b][0], o[b][d], 0, 0, 0);
+            }
+#pragma unroll
+            for (int b = 0; b < QB; b++) o[b][DB] = __builtin_amdgcn_mfma_f32_16x16x16f16(ones4, pf[b][0], o[b][DB], 0, 0, 0);
+        } else {
+#pragma unroll
+        for (int t = 0; t < GKB32; t++) {
 #pragma unroll
             for (int d = 0; d < DB; d++) {
                 half8_t vf = *reinterpret_cast<const half8_t *>(vt_lds + (16 * d + j) * VS +
-                                                                (((4 * t + kb) ^ swz(16 * d + j)) << 3));
+                                                                (((4 * (kgroup * GKB32 + t) + kb) ^ swz(16 * d + j)) << 3));
 #pragma unroll
                 for (int b = 0; b < QB; b++) o[b][d] = mfma16(vf, pf[b][t], o[b][d]);
             }
 #pragma unroll
             for (int b = 0; b < QB; b++) o[b][DB] = mfma16(ones, pf[b][t], o[b][DB]);
         }
+        }
         }   // !PVB
         }   // !skip
+        if (math_first && key0 + BN < keys_scored) {
+            stage(cur ^ 1);
+            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
+        }
         __syncthreads();  // tile i+1 is visible; every wave is done reading tile i
     }
 
     if constexpr (KSPLIT > 1) {
-        // ---- merge the key groups: group 1 hands (m, O, l) to group 0 through LDS (the tile buffers
-        // are free: the loop ended with a barrier), DCH accumulator blocks per pass
-        static_assert(KSPLIT == 2, "two key groups");
+        // ---- merge the key groups: groups 1, 2, ... hand (m, O, l) to group 0 through LDS one after
+        // the other (a fixed order of additions; the tile buffers are free: the loop ended with a
+        // barrier), DCH accumulator blocks per pass
         constexpr int kLdsBytes = kBufHalfs * 2 * 2;
         constexpr int kPerBlock = QWAVES * QB * 64 * 16;                      // bytes of one accumulator block
         constexpr int DCH = (kLdsBytes - QWAVES * QB * 64 * 4) / kPerBlock < DB + 1
@@ -417,36 +461,41 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         static_assert(DCH >= 1, "no room for the merge");
         float *xm = reinterpret_cast<float *>(smem);                          // [QWAVES][QB][64]
         float4_t *xo = reinterpret_cast<float4_t *>(xm + QWAVES * QB * 64);   // [DCH][QWAVES][QB][64]
-        float w0[QB], w1[QB];
 #pragma unroll
-        for (int d0 = 0; d0 <= DB; d0 += DCH) {
-            if (kgroup == 1) {
+        for (int g = 1; g < KSPLIT; g++) {
+            float w0[QB], w1[QB];
 #pragma unroll
-                for (int b = 0; b < QB; b++) {
-                    if (d0 == 0) xm[(qwave * QB + b) * 64 + lane] = m_run[b];
+            for (int d0 = 0; d0 <= DB; d0 += DCH) {
+                if (kgroup == g) {
 #pragma unroll
-                    for (int d = d0; d < d0 + DCH && d <= DB; d++)
-                        xo[(((d - d0) * QWAVES + qwave) * QB + b) * 64 + lane] = o[b][d];
-                }
-            }
-            __syncthreads();
-            if (kgroup == 0) {
+                    for (int b = 0; b < QB; b++) {
+                        if (d0 == 0) xm[(qwave * QB + b) * 64 + lane] = m_run[b];
 #pragma unroll
-                for (int b = 0; b < QB; b++) {
-                    if (d0 == 0) {
-                        const float m1 = xm[(qwave * QB + b) * 64 + lane];
-                        const float m = fmaxf(m_run[b], m1);
-                        w0[b] = __builtin_amdgcn_exp2f((m_run[b] - m) * scale_log2e);
-                        w1[b] = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m1 - m) * scale_log2e);
+                        for (int d = d0; d < d0 + DCH && d <= DB; d++)
+                            xo[(((d - d0) * QWAVES + qwave) * QB + b) * 64 + lane] = o[b][d];
                     }
-#pragma unroll
-                    for (int d = d0; d < d0 + DCH && d <= DB; d++)
-                        o[b][d] = o[b][d] * w0[b] + xo[(((d - d0) * QWAVES + qwave) * QB + b) * 64 + lane] * w1[b];
                 }
+                __syncthreads();
+                if (kgroup == 0) {
+#pragma unroll
+                    for (int b = 0; b < QB; b++) {
+                        if (d0 == 0) {
+                            const float m1 = xm[(qwave * QB + b) * 64 + lane];
+                            const float m = fmaxf(m_run[b], m1);
+                            w0[b] = m_run[b] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m_run[b] - m) * scale_log2e);
+                            w1[b] = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m1 - m) * scale_log2e);
+                            m_run[b] = m;
+                        }
+#pragma unroll
+                        for (int d = d0; d < d0 + DCH && d <= DB; d++)
+                            o[b][d] = o[b][d] * w0[b] + xo[(((d - d0) * QWAVES + qwave) * QB + b) * 64 + lane] * w1[b];
+                    }
+                }
+                // the next pass (of this group or the next one) overwrites the exchange area
+                if (d0 + DCH <= DB || g + 1 < KSPLIT) __syncthreads();
             }
-            if (d0 + DCH <= DB) __syncthreads();   // the next pass overwrites the exchange area
         }
-        if (kgroup == 1) return;
+        if (kgroup != 0) return;
     }
 
     // ---- epilogue: finish the row sums, normalise, store [q][dd]

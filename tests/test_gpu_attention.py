@@ -37,9 +37,13 @@ def _qkv(rng, heads, L, d, mode, orc, ints=False):
 @pytest.mark.parametrize("mode,heads,L,d", [
     ("E5M2", 1, 128, 64), ("E5M2", 3, 256, 64), ("E4M3", 2, 128, 64), ("E5M2", 2, 128, 128),
     ("E4M3", 1, 64, 256), ("E4M3", 1, 96, 512), ("E5M2", 1, 64, 512), ("E5M2", 8, 1024, 64),
-    # d = 256 below 256 workgroups: two wave groups split the key tiles (even, odd and ragged tile counts)
-    ("E4M3", 2, 200, 256), ("E5M2", 1, 330, 256), ("E4M3", 1, 128, 256),
-    ("E4M3", 2, 100, 512), ("E5M2", 1, 200, 512),            # the same split at d = 512 (32-key tiles)
+    # d = 256 below 256 workgroups: two wave groups take one half of every key tile each; the last tile
+    # leaves the second group nothing (200, 330), a few keys (100, 300), everything (128), and a sequence
+    # shorter than the first group's half
+    ("E4M3", 2, 200, 256), ("E5M2", 1, 330, 256), ("E4M3", 1, 128, 256), ("E5M2", 2, 100, 256),
+    ("E4M3", 1, 300, 256), ("E4M3", 1, 7, 256),
+    # the same split at d = 512 (32-key tiles, 16 keys per group on the 16x16x16 MFMA)
+    ("E4M3", 2, 100, 512), ("E5M2", 1, 200, 512), ("E4M3", 1, 50, 512), ("E5M2", 2, 81, 512), ("E4M3", 1, 3, 512),
 ])
 def test_flash_attention_vs_oracle(dev, orc, mode, heads, L, d):
     from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu

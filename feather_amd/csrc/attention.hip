@@ -564,6 +564,9 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
     auto fills_chip = [&](int64_t queries_per_group) {
         return (rows + queries_per_group - 1) / queries_per_group * seqs * a.n_heads >= 256;
     };
+    auto rounds = [&](int64_t queries_per_group) {   // passes of the grid over the 256 CUs, one workgroup per CU
+        return ((rows + queries_per_group - 1) / queries_per_group * seqs * a.n_heads + 255) / 256;
+    };
     switch (d) {
         case 64:   // all four query blocks of a wave share every K fragment
             // eight waves halve the staging work per query (-2 % time); a causal tile of 512 queries
@@ -573,20 +576,25 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
         case 128:
             if (fills_chip(256)) return launch_attn<128, MODE, 2, 2, 64, 1, VC, 8>(a, s);
             return launch_attn<128, MODE, 2, 2, 64, 2, VC>(a, s);
-        case 256:
-            // short sequences: 64 queries per workgroup, the key tiles split between two groups of four
-            // waves (L = 1024: 56.7 -> 48.4 us)
-            if (!a.causal && !fills_chip(128)) return launch_attn<256, MODE, 1, 1, 64, 1, VC, 8, 2>(a, s);
-            // long sequences: 32 queries per wave halve the LDS reads per query, which bound this head dim
-            // (L = 8192: 792 -> 640 us); needs 256 workgroups of 256 queries to cover the chip
-            if (fills_chip(256)) return launch_attn<256, MODE, 2, 2, 32, 1, VC, 8>(a, s);
+        case 256: {
+            // Three shapes, from the finest work items to the cheapest per query (time per 64 keys of
+            // a workgroup's loop at full occupancy, measured): A = 64 queries, two wave groups halve
+            // every key tile (2.9 us); B = 128 queries, eight waves of 16 (3.2 us); C = 256 queries,
+            // eight waves of 32 on 32-key tiles, which halves the LDS reads per query that bound this
+            // head dim (4.6 us; L = 8192: 792 -> 640 us against B).  Pick by rounds over the 256 CUs x cost.
+            const int64_t ra = rounds(64), rb = rounds(128), rc = rounds(256);
+            if (!a.causal && ra * 29 <= rb * 32 && ra * 29 <= rc * 46) return launch_attn<256, MODE, 1, 1, 64, 1, VC, 8, 2>(a, s);
+            if (rc * 46 < rb * 32 || fills_chip(256)) return launch_attn<256, MODE, 2, 2, 32, 1, VC, 8>(a, s);
             return launch_attn<256, MODE, 1, 1, 64, 1, VC, 8>(a, s);
-        case 512:
-            if (fills_chip(128)) return launch_attn<512, MODE, 1, 1, 32, 1, VC, 8>(a, s);
-            // short sequences: 64 queries per workgroup, two groups of four waves alternate over the key tiles
-            // (L = 1024: 129.5 -> 116.3 us)
-            if (!a.causal) return launch_attn<512, MODE, 1, 1, 32, 1, VC, 8, 2>(a, s);
+        }
+        case 512: {
+            // A = 64 queries, two wave groups of 16 keys per 32-key tile (3.1 us per tile of a
+            // workgroup's loop); B = 128 queries, eight waves (3.5 us)
+            const int64_t ra = rounds(64), rb = rounds(128);
+            if (!a.causal && ra * 31 <= rb * 35) return launch_attn<512, MODE, 1, 1, 32, 1, VC, 8, 2>(a, s);
+            if (fills_chip(128) || !a.causal) return launch_attn<512, MODE, 1, 1, 32, 1, VC, 8>(a, s);
             return launch_attn<512, MODE, 1, 1, 32, 1, VC>(a, s);
+        }
     }
     set_error("feather_flash_attn_fp8: head dim %lld not supported (64, 128, 256, 512)", (long long)d);
     return FEATHER_ESHAPE;

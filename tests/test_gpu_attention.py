@@ -75,11 +75,11 @@ def test_flash_attention_reference_signature_and_ints(dev, orc):
     assert np.abs(out.cpu().numpy() - sd.numpy()).max() <= 2e-3
 
 
-@pytest.mark.parametrize("L", [1, 5, 63, 65, 70, 130])
-def test_flash_attention_ragged_tails(dev, orc, L):
+@pytest.mark.parametrize("L,d", [(1, 64), (5, 64), (63, 64), (65, 64), (70, 64), (130, 64),
+                                 (70, 256), (100, 256), (40, 512), (81, 512)])   # wide heads: two key groups per tile
+def test_flash_attention_ragged_tails(dev, orc, L, d):
     from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
     rng = np.random.default_rng(L)
-    d = 64
     q, k, v = _qkv(rng, 2, L, d, "E5M2", orc)
     args = (_dev_words(q, dev), _dev_words(k, dev), _dev_words(v, dev), L, d // 4)
     masked = flash_attention_fp8_acc_fp32_gpu(*args, tail="mask").cpu().numpy()

@@ -91,6 +91,12 @@ def main() -> int:
         bufs, vp = mats[mode], vecs[mode]
         return lambda i: feather.gemv(bufs[i % NBUF], vp, original_shape=(M, K), mode=mode)
 
+    # Clock ramp: the first tens of milliseconds of GPU work in a process run below the sustained clock
+    # (three back-to-back series of 200 launches measured 45.7, 43.9 and 43.0 us), so the same launches
+    # run for ~50 ms before the W warm-up steps; the timed region stays exactly K steps.
+    PREWARM = 1200
+    for i in range(PREWARM):
+        gemv_step("E4M3")(i)
     # the whole timed region, bracketed by synchronize on both sides
     for i in range(args.warmup):
         gemv_step("E4M3")(i)
@@ -133,7 +139,7 @@ def main() -> int:
         del mats["E4M3"]
         torch.cuda.empty_cache()
         mats["E5M2"] = [make_matrix("E5M2") for _ in range(NBUF)]
-        us = gpu_time_us(gemv_step("E5M2"), args.steps, args.warmup, sync)
+        us = gpu_time_us(gemv_step("E5M2"), args.steps, PREWARM + args.warmup, sync)   # same clock pre-warm as the headline
         extra["gemv_e5m2_16384_us"] = round(us, 2)
         extra["gemv_e5m2_16384_GBps"] = round(gemv_bytes / us / 1e3, 1)
         extra["gemv_e5m2_16384_hbm_frac"] = round(gemv_bytes / us / 1e3 / HBM_PEAK_GBS, 4)
@@ -276,7 +282,7 @@ def main() -> int:
         "config": {"workload": "E4M3 packed GEMV 16384x16384 + vector 16384 (the configuration the metric is quoted on); N(0,1) fp16 "
                                "sources with 1% of entries x1e-3, packed 4 codes per 32-bit word; 4 distinct "
                                "matrices (1 GiB) rotated",
-                   "M": M, "K": K, "mode": "E4M3", "buffers": NBUF},
+                   "M": M, "K": K, "mode": "E4M3", "buffers": NBUF, "clock_prewarm_launches": PREWARM},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": "gemv_fp8_kernel<E4M3>", "algorithmic_bytes": gemv_bytes,

@@ -33,7 +33,7 @@
 // bits; 0x7F / 0xFF).  Correct, but the RNE packer emits those subnormal codes
 // for every |x| < 2^-6, 1-2 % of N(0,1) data, so every batch of a wave (8192
 // codes) falls back and pays for both decodes: 64 us.  (6) Per-wave time
-// stamps (s_memrealtime) show that the two waves of a SIMD do not advance
+// stamps (s_memrealtime; one workgroup of 64 rows per CU) show that the two waves of a SIMD do not advance
 // together: the older one wins the vector ALU whenever both have data and ends
 // 6-11 us before the younger one in E4M3 mode (3 us in E5M2), all workgroups
 // ending within 3 us of each other.  Levelling the two through s_setprio (each
@@ -47,8 +47,8 @@
 // modes at 8192^2; with the matrix loads issued first the vector words queue
 // behind them (+2.4 us).
 //
-// A workgroup takes a contiguous range of rows so the vector decode is
-// amortised; ranges are sized so that the grid is a few workgroups per CU.
+// A workgroup takes a contiguous range of rows and decodes the vector once for
+// all of them.
 #include "common.h"
 
 namespace feather {
@@ -199,11 +199,10 @@ __global__ void fill_zero_kernel(float *p, int64_t n) {
 }
 
 template <int MODE, int RPW, int U>
-static int launch_gemv_fast(const void *m, const void *v, float *out, int64_t M, int64_t K, hipStream_t s) {
+static int launch_gemv_fast(const void *m, const void *v, float *out, int64_t M, int64_t K, int64_t wgs, hipStream_t s) {
     constexpr int WAVES = 8;
     constexpr int kStep = kWave * 16;
-    constexpr int kCUs = 256;
-    int64_t rows_per_wg = (M + kCUs - 1) / kCUs;
+    int64_t rows_per_wg = (M + wgs - 1) / wgs;
     rows_per_wg = (rows_per_wg + WAVES * RPW - 1) / (WAVES * RPW) * (WAVES * RPW);
     int64_t blocks = (M + rows_per_wg - 1) / rows_per_wg;
     for (int64_t k0 = 0; k0 < K; k0 += kMaxChunk) {
@@ -233,14 +232,18 @@ static int launch_gemv(const void *m, const void *v, float *out, int64_t M, int6
                            (const uint32_t *)m, (const uint32_t *)v, out, (int)M, K / 4);
         return check_launch("feather_gemv_fp8");
     }
-    // Shape of the launch (measured on MI355X at 16384^2, 4 rotating matrices): one workgroup
-    // of 8 waves per CU, each owning a contiguous range of rows.  E5M2 with long rows: one
-    // row per wave, 4 steps in flight (41.2 us, 81 % of HBM peak).  E4M3, and E5M2 with rows
-    // shorter than 8 steps: four rows per wave share every LDS read of the vector, 2 steps in
-    // flight (E4M3 43.5 us, 77 %).  More waves, deeper unrolling or more workgroups per CU all
-    // measured slower.
-    if (MODE == FEATHER_E5M2 && K >= 8192) return launch_gemv_fast<MODE, 1, 4>(m, v, out, M, K, s);
-    return launch_gemv_fast<MODE, 4, 2>(m, v, out, M, K, s);
+    // Shape of the launch (measured on MI355X, rotating matrices of 1 GiB in total).  Rows of four
+    // steps or more: one row per wave, four steps in flight, and workgroups of eight rows, as many as
+    // the matrix has -- each decodes the vector for itself (1/8 of its matrix bytes, from L2), several
+    // are resident per CU and a CU that finishes one picks up the next, which evens out what one
+    // workgroup per CU with a fixed share of the rows left to the slowest CU.  16384^2: E5M2 41.8 ->
+    // 40.7 us (82 % of the HBM peak), E4M3 45.0 -> 43.0 us (78 %; with one workgroup per CU four rows
+    // per wave that share every LDS read of the vector had been its best shape); 8192^2: 13.0 -> 12.2
+    // and 15.7 -> 13.0 us; 4096 x 8192 E4M3 11.2 -> 8.3 us.  Four-wave or sixteen-wave workgroups, eight
+    // steps in flight and other rotations than 7 steps per row are equal or slower.  Shorter rows keep
+    // four rows per wave and two steps in flight, in twice as many workgroups as CUs.
+    if (K >= 4 * kWave * 16) return launch_gemv_fast<MODE, 1, 4>(m, v, out, M, K, (M + 7) / 8, s);
+    return launch_gemv_fast<MODE, 4, 2>(m, v, out, M, K, 512, s);
 }
 
 }  // namespace feather

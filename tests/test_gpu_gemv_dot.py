@@ -200,6 +200,33 @@ def test_gemv_batched_random_shapes(dev, seed):
     assert ((out.double() - want).abs().max() / scale).item() <= 1e-5
 
 
+@pytest.mark.parametrize("seed", range(14))
+def test_gemv_random_shapes(dev, seed):
+    """Seeded random (mode, M, K) draws for the single-vector GEMV against a float64 matvec of the
+    decoded operands on the device: rows shorter and longer than four 1 KiB steps, ragged last steps,
+    rows longer than one 32768-code vector chunk, row counts that are not a multiple of a workgroup's
+    eight rows, rows that are not 16-byte aligned (generic path); raw random codes."""
+    import feather_amd as feather
+    rng = np.random.default_rng(900 + seed)
+    mode = ("E4M3", "E5M2")[seed % 2]
+    M = int(rng.integers(1, 300))
+    K = int(rng.choice([16, 1024, 2064, 4096, 4112, 5008, 8192, 12304, 32768, 33808, 40000, 65536 + 48, 4 * 77, 4 * 1031]))
+    def codes(n):
+        b = rng.integers(0, 256, size=n, dtype=np.uint8)
+        if mode == "E5M2":
+            b = np.where((b & 0x7C) == 0x7C, b & 0x83, b).astype(np.uint8)   # no inf / NaN codes
+        return torch.from_numpy(b.view(np.int32).copy()).to(dev).view(torch.uint32)
+    wp, xp = codes(M * K), codes(K)
+    print(f"seed {seed}: {mode} M {M} K {K}", flush=True)
+    out = feather.gemv(wp, xp, original_shape=(M, K), mode=mode)
+    wd = feather.unpack_fp8_tensor(wp, mode=mode, semantics="kernel").view(M, K).double()
+    xd = feather.unpack_fp8_tensor(xp, mode=mode, semantics="kernel").view(K).double()
+    want = wd @ xd
+    scale = (wd.abs() @ xd.abs()).max()                 # cancellation-free error scale of the fp32 sums
+    assert out.shape == (M,)
+    assert ((out.double() - want).abs().max() / scale).item() <= 1e-5
+
+
 # ---------------------------------------------------------------- dot
 
 def test_dot_docstring_known_answers(dev, kats):

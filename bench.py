@@ -26,15 +26,23 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_F16_TFLOPS = 2500.0  # dense fp16/bf16, published
+WARM_MS = 40.0                  # warm-up time of the attention series (ours and SDPA alike)
 
 
-def gpu_time_us(fn, steps, warmup, sync):
+def gpu_time_us(fn, steps, warmup, sync, warm_ms=0.0):
     """Average microseconds per call over `steps` back-to-back calls (HIP events on the
-    stream the kernels are launched on: torch's current stream)."""
+    stream the kernels are launched on: torch's current stream).  With `warm_ms` the warm-up calls are
+    repeated until that many milliseconds of back-to-back work have passed: the first tens of
+    milliseconds of a series run below the sustained clock."""
     import torch
+    t0 = time.perf_counter()
     for i in range(warmup):
         fn(i)
     sync()
+    while (time.perf_counter() - t0) * 1000.0 < warm_ms:
+        for i in range(max(warmup, 1)):
+            fn(i)
+        sync()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for i in range(steps):
@@ -178,27 +186,27 @@ def main() -> int:
         del src, words
         del mats["E5M2"], sub, xs
         torch.cuda.empty_cache()
-        # flash attention, B4 H16 d64, E5M2, vs fp16 SDPA on the same GPU (10 warm-up calls each: the
-        # first few milliseconds of a long-kernel series run below the sustained clock)
+        # flash attention, B4 H16 d64, E5M2, vs fp16 SDPA on the same GPU (both sides get WARM_MS of
+        # back-to-back warm-up calls: the first tens of milliseconds of a series run below the sustained clock)
         for L in (4096, 8192):
             B, H, d = 4, 16, 64
             qkv16 = [randn(B, H, L, d).half() for _ in range(3)]
             pk = [feather.pack_fp8_tensor(t, mode="E5M2").view(B, H, L, d // 4) for t in qkv16]
             us = gpu_time_us(lambda i: feather.flash_attention_fp8_e5m2_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4),
-                             10, 10, sync)
+                             10, 10, sync, WARM_MS)
             flops = 4.0 * B * H * L * L * d
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / us / 1e6, 1)
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_mfma_frac"] = round(flops / us / 1e6 / MFMA_PEAK_F16_TFLOPS, 4)
-            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync)
+            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync, WARM_MS)
             extra[f"sdpa_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
             if L == 8192:   # causal prefill (half the flops) vs causal fp16 SDPA
                 us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
-                                                                                    mode="E5M2", causal=True), 10, 10, sync)
+                                                                                    mode="E5M2", causal=True), 10, 10, sync, WARM_MS)
                 extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
                 extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / 2 / us / 1e6, 1)
                 us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16, is_causal=True),
-                                      10, 10, sync)
+                                      10, 10, sync, WARM_MS)
                 extra[f"sdpa_causal_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
             del qkv16, pk
         # wide heads: B1 H8, d = 256 / 512, E4M3, vs fp16 SDPA
@@ -207,10 +215,10 @@ def main() -> int:
             qkv16 = [randn(B, H, L, d).half() for _ in range(3)]
             pk = [feather.pack_fp8_tensor(t, mode="E4M3").view(B, H, L, d // 4) for t in qkv16]
             us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
-                                                                                mode="E4M3"), 10, 10, sync)
+                                                                                mode="E4M3"), 10, 10, sync, WARM_MS)
             extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_us"] = round(us, 1)
             extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_TFLOPs"] = round(4.0 * B * H * L * L * d / us / 1e6, 1)
-            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync)
+            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync, WARM_MS)
             extra[f"sdpa_fp16_b1h8_d{d}_L{L}_us"] = round(us_sdpa, 1)
             del qkv16, pk
         torch.cuda.empty_cache()
@@ -256,7 +264,7 @@ def main() -> int:
             cl = torch.randint(512, cmax, (batch,), generator=g, device=dev, dtype=torch.int32)
             tok = torch.randint(0, cfg.vocab, (batch,), generator=g, device=dev, dtype=torch.int32)
             logits = torch.empty((batch, cfg.vocab), dtype=torch.float32, device=dev)
-            us = gpu_time_us(lambda i: dec.step(tok, btd, cl, out=logits), 20, 10, sync)
+            us = gpu_time_us(lambda i: dec.step(tok, btd, cl, out=logits), 20, 10, sync, WARM_MS)
             step_bytes = dec.weight_bytes() + int(cl.sum().item()) * 2 * cfg.n_kv_heads * cfg.head_dim * cfg.n_layers
             key = f"decode_tinyllama_b{batch}_{mode.lower()}"
             extra[key + "_ms_per_step"] = round(us / 1e3, 3)

@@ -40,12 +40,10 @@
 // wave publishes its step count in LDS, the one behind raises its priority)
 // shrinks that spread to 3 us and leaves the time where it was (43.5 -> 42.8-44.1
 // us): the memory system is as busy with four waves per CU in the last
-// microseconds as with eight.  (7) Fetching the vector with 128-bit loads and the
-// first group of matrix loads before the vector is decoded into LDS (the kernel
-// otherwise starts with two dependent memory latencies, ~2 us): -0.5 us for E5M2
-// at 16384^2 (-1.0 us on uniform random codes), +0.4 us for E4M3 and for both
-// modes at 8192^2; with the matrix loads issued first the vector words queue
-// behind them (+2.4 us).
+// microseconds as with eight.  (7) With one workgroup of 64 rows per CU, fetching the vector with 128-bit
+// loads and the first group of matrix loads before the vector is decoded into LDS
+// gained 0.5 us for E5M2 at 16384^2 only and lost as much elsewhere; it pays since
+// the workgroups are eight rows (see the kernel).
 //
 // A workgroup takes a contiguous range of rows and decodes the vector once for
 // all of them.
@@ -91,52 +89,93 @@ __device__ __forceinline__ float mac16(const u32x4 &a, const u32x4 &x0, const u3
 // worth ~15 % of bandwidth at 16384 x 16384.
 constexpr int kStagger = 7;
 
-template <int MODE, int RPW, int U, int WAVES, bool FULL>
+template <int MODE, int RPW, int U, int WAVES, bool FULL, bool EARLY>
 __global__ __launch_bounds__(WAVES * kWave) void gemv_fp8_kernel(const uint8_t *__restrict__ m,
                                                                 const uint32_t *__restrict__ v,
                                                                 float *__restrict__ out, int M, int64_t K, int k0,
                                                                 int kc, int rows_per_wg, int accumulate) {
     extern __shared__ uint32_t lds32[];  // fp16 vector chunk, zero-padded to whole steps
     constexpr int kStep = kWave * 16;    // codes per wave-load
+    constexpr int kThreads = WAVES * kWave;
     const int n_steps = (kc + kStep - 1) / kStep;
-    for (int i = threadIdx.x; i < n_steps * (kStep / 4); i += WAVES * kWave) {
-        uint32_t p01 = 0, p23 = 0;
-        if (i < kc / 4) dec_word<MODE>(v[i], p01, p23);
-        reinterpret_cast<u32x2 *>(lds32)[i] = u32x2{p01, p23};
-    }
-    __syncthreads();
-
     const int lane = lane_id();
     const int wave = wave_id();
     const int row_begin = blockIdx.x * rows_per_wg;
     const int row_end = min(row_begin + rows_per_wg, M);
-    const u32x4 *lds128 = reinterpret_cast<const u32x4 *>(lds32);
 
+    // One group of wave-loads: U steps of RPW rows, starting at step `it` of the rotated walk.
+    int col[U];
+    u32x4 a[RPW][U];
+    auto issue = [&](int r0, int it) {
+        const int s0 = (int)(((unsigned)(r0 / RPW) * (unsigned)kStagger) % (unsigned)n_steps);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int st = it + u + s0;
+            if (st >= n_steps) st -= n_steps;
+            col[u] = st * kStep;
+#pragma unroll
+            for (int r = 0; r < RPW; r++) {
+                const int row = min(r0 + r, M - 1);  // surplus rows re-read the last row, result dropped
+                if (FULL || col[u] + lane * 16 < kc)
+                    a[r][u] = load_nt128(m + (int64_t)row * K + k0 + lane * 16 + col[u]);
+                else a[r][u] = u32x4{0, 0, 0, 0};
+            }
+        }
+    };
+
+    // The kernel starts with a dependent chain: vector words -> decode -> LDS -> barrier -> first
+    // matrix loads -> first arithmetic, two memory latencies before anything is computed.  With EARLY
+    // a thread fetches its share of the vector (up to kMaxChunk / 16 / kThreads 128-bit loads) and
+    // then at once its first group of matrix loads; loads return in order, so the vector is decoded
+    // into LDS while the matrix data is still on its way.  With workgroups of eight rows, where every
+    // workgroup pays that start for two to four groups of loads: 16384^2 E4M3 43.0 -> 41.15 us, E5M2
+    // 40.9 -> 39.8 us; 8192^2 E5M2 12.14 -> 11.9 us.  (Issued the other way round the vector words
+    // queue behind the matrix loads: slower than no overlap at all.)
+    bool have = false;
+    if (EARLY) {
+        constexpr int kQuads = kMaxChunk / 16 / kThreads;
+        u32x4 xv[kQuads];
+#pragma unroll
+        for (int j = 0; j < kQuads; j++) {
+            const int q = threadIdx.x + j * kThreads;
+            xv[j] = q < kc / 16 ? reinterpret_cast<const u32x4 *>(v)[q] : u32x4{0, 0, 0, 0};
+        }
+        if (n_steps >= U && row_begin + wave * RPW < row_end) {
+            issue(row_begin + wave * RPW, 0);
+            have = true;
+        }
+#pragma unroll
+        for (int j = 0; j < kQuads; j++) {
+            const int q = threadIdx.x + j * kThreads;
+            if (q < n_steps * (kStep / 16)) {
+                uint32_t o[8];
+                dec_word<MODE>(xv[j].x, o[0], o[1]);
+                dec_word<MODE>(xv[j].y, o[2], o[3]);
+                dec_word<MODE>(xv[j].z, o[4], o[5]);
+                dec_word<MODE>(xv[j].w, o[6], o[7]);
+                u32x4 *dst = reinterpret_cast<u32x4 *>(lds32) + 2 * q;
+                dst[0] = u32x4{o[0], o[1], o[2], o[3]};
+                dst[1] = u32x4{o[4], o[5], o[6], o[7]};
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < n_steps * (kStep / 4); i += kThreads) {
+            uint32_t p01 = 0, p23 = 0;
+            if (i < kc / 4) dec_word<MODE>(v[i], p01, p23);
+            reinterpret_cast<u32x2 *>(lds32)[i] = u32x2{p01, p23};
+        }
+    }
+    __syncthreads();
+
+    const u32x4 *lds128 = reinterpret_cast<const u32x4 *>(lds32);
     for (int r0 = row_begin + wave * RPW; r0 < row_end; r0 += WAVES * RPW) {
         float acc[RPW];
-        const uint8_t *rowp[RPW];
 #pragma unroll
-        for (int r = 0; r < RPW; r++) {
-            acc[r] = 0.f;
-            int row = min(r0 + r, M - 1);  // surplus rows re-read the last row, result dropped
-            rowp[r] = m + (int64_t)row * K + k0 + lane * 16;
-        }
-        const int s0 = (int)(((unsigned)(r0 / RPW) * (unsigned)kStagger) % (unsigned)n_steps);
+        for (int r = 0; r < RPW; r++) acc[r] = 0.f;
         int it = 0;
         for (; it + U <= n_steps; it += U) {   // U wave-loads per row in flight
-            int col[U];
-            u32x4 a[RPW][U];
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                int st = it + u + s0;
-                if (st >= n_steps) st -= n_steps;
-                col[u] = st * kStep;
-#pragma unroll
-                for (int r = 0; r < RPW; r++) {
-                    if (FULL || col[u] + lane * 16 < kc) a[r][u] = load_nt128(rowp[r] + col[u]);
-                    else a[r][u] = u32x4{0, 0, 0, 0};
-                }
-            }
+            if (!EARLY || !have) issue(r0, it);
+            have = false;
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 int c8 = (col[u] + lane * 16) / 8;
@@ -145,20 +184,24 @@ __global__ __launch_bounds__(WAVES * kWave) void gemv_fp8_kernel(const uint8_t *
                 for (int r = 0; r < RPW; r++) acc[r] = mac16<MODE>(a[r][u], x0, x1, acc[r]);
             }
         }
-        for (; it < n_steps; it++) {           // fewer than U steps left
-            int st = it + s0;
-            if (st >= n_steps) st -= n_steps;
-            int c = st * kStep;
-            u32x4 a[RPW];
+        if (it < n_steps) {
+            const int s0 = (int)(((unsigned)(r0 / RPW) * (unsigned)kStagger) % (unsigned)n_steps);
+            for (; it < n_steps; it++) {       // fewer than U steps left
+                int st = it + s0;
+                if (st >= n_steps) st -= n_steps;
+                int c = st * kStep;
+                u32x4 b[RPW];
 #pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                if (FULL || c + lane * 16 < kc) a[r] = load_nt128(rowp[r] + c);
-                else a[r] = u32x4{0, 0, 0, 0};
+                for (int r = 0; r < RPW; r++) {
+                    const int row = min(r0 + r, M - 1);
+                    if (FULL || c + lane * 16 < kc) b[r] = load_nt128(m + (int64_t)row * K + k0 + lane * 16 + c);
+                    else b[r] = u32x4{0, 0, 0, 0};
+                }
+                int c8 = (c + lane * 16) / 8;
+                u32x4 x0 = lds128[c8], x1 = lds128[c8 + 1];
+#pragma unroll
+                for (int r = 0; r < RPW; r++) acc[r] = mac16<MODE>(b[r], x0, x1, acc[r]);
             }
-            int c8 = (c + lane * 16) / 8;
-            u32x4 x0 = lds128[c8], x1 = lds128[c8 + 1];
-#pragma unroll
-            for (int r = 0; r < RPW; r++) acc[r] = mac16<MODE>(a[r], x0, x1, acc[r]);
         }
 #pragma unroll
         for (int r = 0; r < RPW; r++) {
@@ -198,7 +241,7 @@ __global__ void fill_zero_kernel(float *p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.f;
 }
 
-template <int MODE, int RPW, int U>
+template <int MODE, int RPW, int U, bool EARLY>
 static int launch_gemv_fast(const void *m, const void *v, float *out, int64_t M, int64_t K, int64_t wgs, hipStream_t s) {
     constexpr int WAVES = 8;
     constexpr int kStep = kWave * 16;
@@ -209,14 +252,20 @@ static int launch_gemv_fast(const void *m, const void *v, float *out, int64_t M,
         int kc = (int)((K - k0) < kMaxChunk ? (K - k0) : kMaxChunk);
         int n_steps = (kc + kStep - 1) / kStep;
         size_t lds = (size_t)n_steps * kStep * 2;
-        if (kc % kStep == 0)
-            hipLaunchKernelGGL((gemv_fp8_kernel<MODE, RPW, U, WAVES, true>), dim3((unsigned)blocks),
-                               dim3(WAVES * kWave), lds, s, (const uint8_t *)m, (const uint32_t *)v + k0 / 4, out,
-                               (int)M, K, (int)k0, kc, (int)rows_per_wg, k0 > 0 ? 1 : 0);
-        else
-            hipLaunchKernelGGL((gemv_fp8_kernel<MODE, RPW, U, WAVES, false>), dim3((unsigned)blocks),
-                               dim3(WAVES * kWave), lds, s, (const uint8_t *)m, (const uint32_t *)v + k0 / 4, out,
-                               (int)M, K, (int)k0, kc, (int)rows_per_wg, k0 > 0 ? 1 : 0);
+        const void *vk = (const uint32_t *)v + k0 / 4;
+        auto go = [&](auto kern) {
+            hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(WAVES * kWave), lds, s, (const uint8_t *)m,
+                               (const uint32_t *)vk, out, (int)M, K, (int)k0, kc, (int)rows_per_wg, k0 > 0 ? 1 : 0);
+        };
+        // E4M3 with rows under 16 steps loses ~1 % with it (measured at K = 8192); the fetch uses 128-bit loads
+        const bool early = EARLY && aligned(vk, 16) && (MODE == FEATHER_E5M2 || kc >= 16 * kStep);
+        if (kc % kStep == 0) {
+            if (early) go(gemv_fp8_kernel<MODE, RPW, U, WAVES, true, EARLY>);
+            else go(gemv_fp8_kernel<MODE, RPW, U, WAVES, true, false>);
+        } else {
+            if (early) go(gemv_fp8_kernel<MODE, RPW, U, WAVES, false, EARLY>);
+            else go(gemv_fp8_kernel<MODE, RPW, U, WAVES, false, false>);
+        }
         int rc = check_launch("feather_gemv_fp8");
         if (rc != FEATHER_OK) return rc;
     }
@@ -237,13 +286,13 @@ static int launch_gemv(const void *m, const void *v, float *out, int64_t M, int6
     // the matrix has -- each decodes the vector for itself (1/8 of its matrix bytes, from L2), several
     // are resident per CU and a CU that finishes one picks up the next, which evens out what one
     // workgroup per CU with a fixed share of the rows left to the slowest CU.  16384^2: E5M2 41.8 ->
-    // 40.7 us (82 % of the HBM peak), E4M3 45.0 -> 43.0 us (78 %; with one workgroup per CU four rows
-    // per wave that share every LDS read of the vector had been its best shape); 8192^2: 13.0 -> 12.2
+    // 40.9 us, E4M3 45.0 -> 43.0 us before the early fetch (with one workgroup per CU four rows
+    // per wave that share every LDS read of the vector had been E4M3's best shape); 8192^2: 13.0 -> 12.2
     // and 15.7 -> 13.0 us; 4096 x 8192 E4M3 11.2 -> 8.3 us.  Four-wave or sixteen-wave workgroups, eight
     // steps in flight and other rotations than 7 steps per row are equal or slower.  Shorter rows keep
     // four rows per wave and two steps in flight, in twice as many workgroups as CUs.
-    if (K >= 4 * kWave * 16) return launch_gemv_fast<MODE, 1, 4>(m, v, out, M, K, (M + 7) / 8, s);
-    return launch_gemv_fast<MODE, 4, 2>(m, v, out, M, K, 512, s);
+    if (K >= 4 * kWave * 16) return launch_gemv_fast<MODE, 1, 4, true>(m, v, out, M, K, (M + 7) / 8, s);
+    return launch_gemv_fast<MODE, 4, 2, false>(m, v, out, M, K, 512, s);
 }
 
 }  // namespace feather

@@ -296,14 +296,16 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                     for (int r = 0; r < 4; r++)
                         if (16 * c + r > rel) sb[c][r] = -INFINITY;
             }
-            float mx = sb[0][0];
+            float mx = max3_raw(sb[0][0], sb[0][1], sb[0][2]);
+            mx = max_raw(mx, sb[0][3]);
 #pragma unroll
-            for (int c = 0; c < GKB16; c++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) mx = fmaxf(mx, sb[c][r]);
+            for (int c = 1; c < GKB16; c++) {
+                mx = max3_raw(mx, sb[c][0], sb[c][1]);
+                mx = max3_raw(mx, sb[c][2], sb[c][3]);
+            }
             mx = max_xor32(max_xor16(mx));   // over the four lanes that share the query
             const float m_old = m_run[qb];
-            const float m_new = fmaxf(m_old, mx);
+            const float m_new = max_raw(m_old, mx);
             const float mc = m_new * scale_log2e;
             if constexpr (K16) {
                 half4_t p4;

@@ -234,6 +234,21 @@ __device__ __forceinline__ float max_xor32(float x) {
     return a;
 }
 
+// max of two / three floats as single instructions.  In front of fmaxf the compiler puts a canonicalising
+// max(x, x) on every value whose NaN quietness it cannot prove (MFMA results, values that came out of
+// inline asm): 4 of the ~80 vector instructions of a softmax block.  Scores are never signalling
+// NaNs, and for quiet NaNs v_max returns the other operand, as fmaxf does.
+__device__ __forceinline__ float max_raw(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }
 
 // Index of the wave inside its workgroup, marked as wave-uniform: everything derived from it (row

@@ -253,10 +253,10 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
                 for (int r = 0; r < 4; r++)
                     if (16 * a + r >= rel) s[a][r] = -INFINITY;
         }
-        float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
-                         fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+        float mx = max3_raw(max3_raw(s[0][0], s[0][1], s[0][2]), s[0][3], s[1][0]);
+        mx = max_raw(max3_raw(mx, s[1][1], s[1][2]), s[1][3]);
         mx = max_xor32(max_xor16(mx));
-        const float m_new = fmaxf(m_run, mx * scale_log2e);      // scale > 0: the maximum commutes with it
+        const float m_new = max_raw(m_run, mx * scale_log2e);    // scale > 0: the maximum commutes with it
         half8_t p8;
         float rs = 0.f;
 #pragma unroll

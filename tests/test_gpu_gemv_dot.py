@@ -227,6 +227,27 @@ def test_gemv_random_shapes(dev, seed):
     assert ((out.double() - want).abs().max() / scale).item() <= 1e-5
 
 
+@pytest.mark.parametrize("mode", ["E5M2", "E4M3"])
+def test_gemv_vector_and_matrix_at_word_offsets(dev, mode):
+    """Operands that are only 4-byte aligned (views one word into a buffer): the vector then takes the
+    word-wise staging path, the matrix the generic kernel; results equal the aligned call bit for bit
+    for the vector case (same summation order) and to fp32 rounding for the matrix case."""
+    import feather_amd as feather
+    g = torch.Generator(device=dev).manual_seed(7)
+    M, K = 40, 16384
+    w = feather.pack_fp8_tensor(torch.randn(M, K, generator=g, device=dev).half(), mode=mode)
+    x = feather.pack_fp8_tensor(torch.randn(K, generator=g, device=dev).half(), mode=mode)
+    want = feather.gemv(w, x, original_shape=(M, K), mode=mode)
+    xbuf = torch.zeros(x.numel() + 1, dtype=x.dtype, device=dev)
+    xbuf[1:].copy_(x)
+    assert xbuf[1:].data_ptr() % 16 == 4
+    assert torch.equal(feather.gemv(w, xbuf[1:], original_shape=(M, K), mode=mode), want)
+    wbuf = torch.zeros(w.numel() + 1, dtype=w.dtype, device=dev)
+    wbuf[1:].copy_(w)
+    got = feather.gemv(wbuf[1:], x, original_shape=(M, K), mode=mode)
+    assert ((got - want).abs().max() / want.abs().max()).item() <= 1e-5
+
+
 # ---------------------------------------------------------------- dot
 
 def test_dot_docstring_known_answers(dev, kats):

@@ -342,7 +342,9 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         // exponentials (d = 64, L = 8192: 1189 -> 1147 us).  The fp16 score path has no registers left
         // for resident K fragments (spills) and re-reading them from LDS per block costs more than the
         // overlap gains (1250 -> 1262 / 1275 us), so there, and for the wider heads, all blocks share
-        // each K / V^T fragment as it is read from LDS.
+        // each K / V^T fragment as it is read from LDS.  (s_setprio 1 around the MFMA groups, or around
+        // the softmax instead, to steer which of a SIMD's two waves issues: 1163 / 1182 us against 1143;
+        // and a run that skipped every other tile barrier, wrong results, was only 1.2 % faster.)
         constexpr bool PVB = KSPLIT == 1 && BF8 && QB > 1 && DB * KB32 <= 8 && KB16 * STEPS <= 8;
         if constexpr (PVB) {
             long kres[KB16][STEPS];

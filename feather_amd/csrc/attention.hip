@@ -25,7 +25,8 @@
 //
 // E5M2 is the matrix core's bf8 operand format, so in that mode S^T runs on
 // v_mfma_f32_16x16x32_bf8_bf8 straight from the packed K and Q bytes (no decode
-// of K, half the LDS bytes, twice the MFMA rate); the products are the same
+// of K, half the LDS bytes; the instruction takes the same 16 cycles as the fp16
+// one, as SQ_VALU_MFMA_BUSY_CYCLES shows); the products are the same
 // exact fp16 x fp16 products, accumulated in fp32.
 //
 // Numerics follow the reference kernel (feather/routines/attention.py:24-108):
@@ -80,7 +81,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     constexpr int DW = D / 4;              // packed words per row
     // E5M2 codes ARE the bf8 operand format of the matrix core: the score product runs on
     // v_mfma_f32_16x16x32_bf8_bf8 straight from the packed bytes (exact products, fp32 accumulation,
-    // twice the fp16 MFMA rate, no decode, half the LDS bytes for K); V still goes through fp16
+    // no decode, half the LDS bytes for K); V still goes through fp16
     // because P is an fp16 operand (the reference rounds P to fp16, attention.py:90).
     constexpr bool BF8 = MODE == FEATHER_E5M2;
     constexpr int KS = BF8 ? (D + 16) / 2 : D + 8;   // K row pitch in LDS, in fp16 units (bf8: D + 16 bytes)

@@ -22,6 +22,7 @@ namespace feather {
 
 constexpr int kDsThreads = 256;
 
+template <int THREADS = kDsThreads>
 __device__ __forceinline__ float block_sum(float x, float *red) {
     x = wave_sum(x);
     const int lane = lane_id(), wave = wave_id();
@@ -29,7 +30,7 @@ __device__ __forceinline__ float block_sum(float x, float *red) {
     __syncthreads();
     float t = 0.f;
 #pragma unroll
-    for (int w = 0; w < kDsThreads / kWave; w++) t += red[w];
+    for (int w = 0; w < THREADS / kWave; w++) t += red[w];
     __syncthreads();
     return t;
 }
@@ -67,25 +68,25 @@ __device__ __forceinline__ float4 load_parts(const float *p, int n_part, int64_t
 // 4096 elements (h, the norm weights and up to eight partial sums per element) is issued before
 // the first value is used, and the second pass works from registers: two round trips (loads,
 // stores) instead of one per 1024 elements and pass.
-template <int MODE>
-__global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__restrict__ h,
+template <int MODE, int KEEP, int THREADS>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_pack_kernel(float *__restrict__ h,
                                                                      const float *__restrict__ delta, int n_part,
                                                                      int64_t part_stride,
                                                                      const float *__restrict__ w,
                                                                      uint32_t *__restrict__ xq, int hidden,
                                                                      float eps) {
-    __shared__ float red[kDsThreads / kWave];
+    __shared__ float red[THREADS / kWave];
     const int b = blockIdx.x;
     float4 *hr = reinterpret_cast<float4 *>(h + (int64_t)b * hidden);
     const float *dr = delta ? delta + (int64_t)b * hidden : nullptr;
     const float4 *wr = reinterpret_cast<const float4 *>(w);
     const int n4 = hidden / 4;
-    constexpr int kKeep = 4, G = 8;
+    constexpr int kKeep = KEEP, G = 8;
     float4 x[kKeep], g[kKeep], part[kKeep][G];
     // ---- all loads (inactive slots read element 0 and are dropped)
 #pragma unroll
     for (int it = 0; it < kKeep; it++) {
-        const int i = threadIdx.x + it * kDsThreads, ii = i < n4 ? i : 0;
+        const int i = threadIdx.x + it * THREADS, ii = i < n4 ? i : 0;
         x[it] = hr[ii];
         g[it] = wr[ii];
         if (dr) {
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__r
     float ss = 0.f;
 #pragma unroll
     for (int it = 0; it < kKeep; it++) {
-        const int i = threadIdx.x + it * kDsThreads;
+        const int i = threadIdx.x + it * THREADS;
         if (i < n4) {
             if (dr) {
                 float4 d = part[it][0];                      // slices are added in index order
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__r
             ss += (x[it].x * x[it].x + x[it].y * x[it].y) + (x[it].z * x[it].z + x[it].w * x[it].w);
         }
     }
-    for (int i = threadIdx.x + kKeep * kDsThreads; i < n4; i += kDsThreads) {   // rows longer than 4096
+    for (int i = threadIdx.x + kKeep * THREADS; i < n4; i += THREADS) {   // rows longer than 4096
         float4 y = hr[i];
         if (dr) {
             float4 d = load_parts(dr + 4 * i, n_part, part_stride);
@@ -128,21 +129,40 @@ __global__ __launch_bounds__(kDsThreads) void add_rmsnorm_pack_kernel(float *__r
         }
         ss += (y.x * y.x + y.y * y.y) + (y.z * y.z + y.w * y.w);
     }
-    const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
+    const float r = 1.0f / sqrtf(block_sum<THREADS>(ss, red) / (float)hidden + eps);
 #pragma unroll
     for (int it = 0; it < kKeep; it++) {
-        const int i = threadIdx.x + it * kDsThreads;
+        const int i = threadIdx.x + it * THREADS;
         if (i < n4)
             xq[(int64_t)b * n4 + i] = quant4<MODE>(x[it].x * r * g[it].x, x[it].y * r * g[it].y, x[it].z * r * g[it].z,
                                                   x[it].w * r * g[it].w);
     }
-    for (int i = threadIdx.x + kKeep * kDsThreads; i < n4; i += kDsThreads) {
+    for (int i = threadIdx.x + kKeep * THREADS; i < n4; i += THREADS) {
         float4 y = hr[i], gg = wr[i];
         xq[(int64_t)b * n4 + i] = quant4<MODE>(y.x * r * gg.x, y.y * r * gg.y, y.z * r * gg.z, y.w * r * gg.w);
     }
 }
 
 // gu [B, 2 * inter] (gate rows then up rows) -> pack(fp16(silu(gate) * up)) [B, inter / 4]
+// One workgroup per vector; the row is spread over as many threads as it has groups of four elements (up to
+// 512), so a thread issues the loads of one group -- residual, gain, eight partial sums -- instead of
+// several: the kernel is one memory round trip plus a block reduction, and its length is the time the
+// workgroup's loads take to drain through one CU (TinyLlama width, 256 threads with two groups each
+// and two idle slots: 2.1 us from entry to the sums; see the launcher of the decode step).
+template <int MODE>
+static void launch_norm(int batch, hipStream_t s, float *h, const float *delta, int n_part, int64_t part_stride,
+                        const void *w, uint32_t *xq, int hidden, float eps) {
+    const int n4 = hidden / 4;
+    auto go = [&](auto kern, int threads) {
+        hipLaunchKernelGGL(kern, dim3(batch), dim3(threads), 0, s, h, delta, n_part, part_stride, (const float *)w, xq,
+                           hidden, eps);
+    };
+    if (n4 <= 256) go(add_rmsnorm_pack_kernel<MODE, 1, 256>, 256);
+    else if (n4 <= 512) go(add_rmsnorm_pack_kernel<MODE, 1, 512>, 512);
+    else if (n4 <= 1024) go(add_rmsnorm_pack_kernel<MODE, 2, 512>, 512);
+    else go(add_rmsnorm_pack_kernel<MODE, 4, 512>, 512);
+}
+
 template <int MODE>
 __global__ __launch_bounds__(kDsThreads) void swiglu_pack_kernel(const float *__restrict__ gu, int n_part,
                                                                 int64_t part_stride,
@@ -332,8 +352,7 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
     const int64_t hs = (int64_t)batch * H;
     for (int l = 0; l < dec->n_layers; l++) {
         const feather_decoder_layer_t &L = dec->layers[l];
-        hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending, P.s_down, hs,
-                           L.norm_attn, xq, H, dec->rms_eps);
+        launch_norm<MODE>(batch, s, h, pending, P.s_down, hs, L.norm_attn, xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
         DS_CHECK(gemv(L.w_qkv, qkv, qkv_rows, H, P.s_qkv));
         hipLaunchKernelGGL((rope_append_kernel<MODE>),
@@ -345,8 +364,7 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
         DS_CHECK(paged_attn_launch(qp, L.k_cache, L.v_cache, block_tables, ctx_after, nullptr, xq, nullptr, pa_scratch, batch, nq,
                                    nkv, d, dec->block_size, dec->max_blocks, max_ctx, MODE, scale, s));
         DS_CHECK(gemv(L.w_o, delta, H, nq * d, P.s_o));
-        hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, delta, P.s_o, hs,
-                           L.norm_mlp, xq, H, dec->rms_eps);
+        launch_norm<MODE>(batch, s, h, delta, P.s_o, hs, L.norm_mlp, xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
         if (P.fused_mlp) {
             DS_CHECK(gemv_batched_swiglu_launch(L.w_gate_up, xq, act, I, H, batch, MODE, s));
@@ -360,8 +378,7 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
         DS_CHECK(gemv_x(L.w_down, act, delta, H, I, P.s_down));
         pending = delta;
     }
-    hipLaunchKernelGGL((add_rmsnorm_pack_kernel<MODE>), dim3(batch), dim3(kDsThreads), 0, s, h, pending, P.s_down, hs,
-                       dec->norm_final, xq, H, dec->rms_eps);
+    launch_norm<MODE>(batch, s, h, pending, P.s_down, hs, dec->norm_final, xq, H, dec->rms_eps);
     DS_CHECK(check_launch("feather_decode_step (final norm)"));
     DS_CHECK(feather_gemv_fp8_batched(dec->w_lm_head, xq, logits, dec->vocab, H, batch, MODE, st));
 #undef DS_CHECK

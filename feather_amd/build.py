@@ -30,6 +30,10 @@ HIPCC_FLAGS = [
     # MFMA accumulators stay in architectural VGPRs: the kernels rescale them with VALU ops, and
     # every such touch of an AGPR accumulator costs a v_accvgpr_read/write pair
     "-mllvm", "-amdgpu-mfma-vgpr-form",
+    # the first 16 dwords of kernel arguments arrive in SGPRs with the wave instead of through s_load
+    # (a cold scalar-cache miss at the start of every kernel); code objects keep a loader prologue for
+    # firmware without the feature
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-function",
 ]
 

@@ -199,17 +199,17 @@ __device__ __forceinline__ void sincos_small(float x, float &s, float &c) {
     c = ((q + 1) & 2) ? -cc : cc;
 }
 
+// (parameter order: everything needed before the first loads sits in the 16 preloaded dwords)
 template <int MODE>
-__global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *__restrict__ qkv, int n_part,
-                                                                int64_t part_stride,
-                                                                uint32_t *__restrict__ qp,
+__global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *__restrict__ qkv,
+                                                                const int32_t *__restrict__ ctx_lens,
+                                                                const int32_t *__restrict__ block_tables,
+                                                                int64_t part_stride, int n_part, int n_q, int n_kv,
+                                                                int d, int block_size, int max_blocks,
+                                                                float log2_theta, uint32_t *__restrict__ qp,
                                                                 uint32_t *__restrict__ k_cache,
                                                                 uint32_t *__restrict__ v_cache,
-                                                                const int32_t *__restrict__ block_tables,
-                                                                const int32_t *__restrict__ ctx_lens,
-                                                                int32_t *__restrict__ ctx_after, int n_q, int n_kv,
-                                                                int d, int block_size, int max_blocks,
-                                                                float log2_theta) {
+                                                                int32_t *__restrict__ ctx_after) {
     const int b = blockIdx.x;
     const int dw = d / 4, half_w = d / 8;            // words per head, words per rotation half
     const int heads = n_q + 2 * n_kv;
@@ -373,9 +373,9 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
         DS_CHECK(check_launch("feather_decode_step (norm)"));
         DS_CHECK(gemv(L.w_qkv, qkv, qkv_rows, H, P.s_qkv));
         hipLaunchKernelGGL((rope_append_kernel<MODE>),
-                           dim3(batch, ((nq + 2 * nkv) * (d / 8) + kRopeThreads - 1) / kRopeThreads), dim3(kRopeThreads), 0, s, qkv, P.s_qkv,
-                           (int64_t)batch * qkv_rows, qp, (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, block_tables,
-                           ctx_lens, ctx_after, nq, nkv, d, dec->block_size, dec->max_blocks, log2_theta);
+                           dim3(batch, ((nq + 2 * nkv) * (d / 8) + kRopeThreads - 1) / kRopeThreads), dim3(kRopeThreads), 0, s, qkv, ctx_lens,
+                           block_tables, (int64_t)batch * qkv_rows, P.s_qkv, nq, nkv, d, dec->block_size, dec->max_blocks,
+                           log2_theta, qp, (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, ctx_after);
         DS_CHECK(check_launch("feather_decode_step (rope)"));
         // attention writes its output already rounded to FP8 and packed (the operand of W_o)
         DS_CHECK(paged_attn_launch(qp, L.k_cache, L.v_cache, block_tables, ctx_after, nullptr, xq, nullptr, pa_scratch, batch, nq,

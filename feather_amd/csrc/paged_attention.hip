@@ -70,12 +70,16 @@ __device__ __forceinline__ void v_pairs(uint32_t wa, uint32_t wb, uint32_t out[4
 // scratch per (seq, q head, split): [0] = m (log2 domain), [1] = l, [2 .. 2+D) = unnormalised O
 // FAST: block_size is a power of two >= 4: token -> block / slot by shift and mask, and an aligned
 // group of 4 tokens never straddles a block (one table lookup per group)
+// (parameter order: what a wave needs before its first loads -- the lengths, the table, the operands
+// and the shape -- fills the 16 dwords of kernel arguments that arrive preloaded in SGPRs; the rest
+// is fetched with s_load while those loads are in flight)
 template <int D, int MODE, bool FAST>
 __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
-    const uint32_t *__restrict__ q, const uint32_t *__restrict__ k_cache, const uint32_t *__restrict__ v_cache,
-    const int32_t *__restrict__ block_tables, const int32_t *__restrict__ ctx_lens, float *__restrict__ scratch,
-    float *__restrict__ out_f32, uint32_t *__restrict__ out_packed, _Float16 *__restrict__ out_q16, int n_q_heads,
-    int n_kv_heads, int block_size, int bs_shift, int max_blocks, int n_splits, int max_ctx, float scale_log2e) {
+    const int32_t *__restrict__ ctx_lens, const int32_t *__restrict__ block_tables, const uint32_t *__restrict__ q,
+    const uint32_t *__restrict__ k_cache, const uint32_t *__restrict__ v_cache, int n_q_heads, int n_kv_heads,
+    int block_size, int max_blocks, int n_splits, int max_ctx, float scale_log2e, float *__restrict__ scratch,
+    float *__restrict__ out_f32, uint32_t *__restrict__ out_packed, _Float16 *__restrict__ out_q16) {
+    const int bs_shift = FAST ? __builtin_ctz((unsigned)block_size) : 0;
     constexpr int DW = D / 4;       // words per token row
     constexpr int RB = D / 64;      // 16-word row blocks of V per token
     constexpr int STEPS = D / 32;   // MFMA k-steps of the score product
@@ -444,14 +448,14 @@ static int launch_paged(const void *q, const void *kc, const void *vc, const voi
     const float log2e = 1.4426950408889634f;
     if (bs_shift >= 2)
         hipLaunchKernelGGL((paged_attn_split_kernel<D, MODE, true>), dim3((unsigned)blocks), dim3(kPaThreads), 0, s,
-                           (const uint32_t *)q, (const uint32_t *)kc, (const uint32_t *)vc, (const int32_t *)bt,
-                           (const int32_t *)cl, (float *)scratch, out_f32, out_packed, out_q16, (int)n_q_heads, (int)n_kv_heads,
-                           (int)block_size, bs_shift, (int)max_blocks, n_splits, (int)max_ctx, scale * log2e);
+                           (const int32_t *)cl, (const int32_t *)bt, (const uint32_t *)q, (const uint32_t *)kc,
+                           (const uint32_t *)vc, (int)n_q_heads, (int)n_kv_heads, (int)block_size, (int)max_blocks, n_splits,
+                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16);
     else
         hipLaunchKernelGGL((paged_attn_split_kernel<D, MODE, false>), dim3((unsigned)blocks), dim3(kPaThreads), 0, s,
-                           (const uint32_t *)q, (const uint32_t *)kc, (const uint32_t *)vc, (const int32_t *)bt,
-                           (const int32_t *)cl, (float *)scratch, out_f32, out_packed, out_q16, (int)n_q_heads, (int)n_kv_heads,
-                           (int)block_size, bs_shift, (int)max_blocks, n_splits, (int)max_ctx, scale * log2e);
+                           (const int32_t *)cl, (const int32_t *)bt, (const uint32_t *)q, (const uint32_t *)kc,
+                           (const uint32_t *)vc, (int)n_q_heads, (int)n_kv_heads, (int)block_size, (int)max_blocks, n_splits,
+                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16);
     int rc = check_launch("feather_paged_attn_fp8");
     if (rc != FEATHER_OK || n_splits == 1) return rc;
     int64_t threads = n_seq * n_q_heads * (D / 4);

@@ -173,7 +173,10 @@ __global__ __launch_bounds__(kDsThreads) void swiglu_pack_kernel(const float *__
         int b = (int)(i / per_row), c = (int)(i % per_row);
         float4 g = load_parts(gu + (int64_t)b * 2 * inter + 4 * c, n_part, part_stride);
         float4 u = load_parts(gu + (int64_t)b * 2 * inter + inter + 4 * c, n_part, part_stride);
-        auto f = [](float a, float bb) { return a / (1.0f + expf(-a)) * bb; };
+        // the same arithmetic as the fused epilogue of the gate/up GEMV
+        auto f = [](float a, float bb) {
+            return a * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * a)) * bb;
+        };
         out[i] = quant4<MODE>(f(g.x, u.x), f(g.y, u.y), f(g.z, u.z), f(g.w, u.w));
     }
 }

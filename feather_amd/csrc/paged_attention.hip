@@ -101,9 +101,44 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     if (n_splits > 1) {
         const int n_seq = gridDim.x / (n_splits * n_kv_heads);
         const int item = blockIdx.x / n_kv_heads;          // index over the (sequence, split) pairs that exist
-        int base = 0;
         seq = -1;
         ctx_raw = 0;
+        if (n_seq <= kWave) {
+            // Largest items first: all full splits in sequence order, then the partial last splits by
+            // size, largest first.  Every workgroup with work is resident at once and the hardware deals
+            // them to the CUs in launch order, so when the items are not a multiple of the CUs the CUs
+            // that get one more than the others get the smallest ones (with sequence order a full split
+            // could be the extra one and its CU finished last: 15 us against 10 us for the median).
+            const int c = lane < n_seq ? max(ctx_lens[lane], 0) : 0;
+            const int cc = min(c, max_ctx);
+            const int nf = cc / kSplit, ps = cc % kSplit;   // full splits, tokens of the partial one
+            int inc = nf;                                   // inclusive prefix sum over the lanes
+#pragma unroll
+            for (int off = 1; off < kWave; off <<= 1) {
+                const int t = __shfl_up(inc, off, kWave);
+                if (lane >= off) inc += t;
+            }
+            const int n_full = __builtin_amdgcn_readlane(inc, kWave - 1);
+            uint64_t hit;
+            if (item < n_full) {
+                const int exc = inc - nf;
+                hit = __builtin_amdgcn_ballot_w64(item >= exc && item < exc + nf);
+                if (hit) split = item - __builtin_amdgcn_readlane(exc, __builtin_ctzll(hit));
+            } else {
+                int rank = 0;                               // partial splits larger than this lane's (ties: lower sequence first)
+                for (int t = 0; t < n_seq; t++) {
+                    const int pt = __builtin_amdgcn_readlane(ps, t);
+                    rank += (pt > ps || (pt == ps && t < lane)) ? 1 : 0;
+                }
+                hit = __builtin_amdgcn_ballot_w64(ps > 0 && rank == item - n_full);
+                if (hit) split = __builtin_amdgcn_readlane(nf, __builtin_ctzll(hit));
+            }
+            if (hit) {
+                seq = __builtin_ctzll(hit);
+                ctx_raw = __builtin_amdgcn_readlane(c, seq);
+            }
+        } else {
+        int base = 0;
         for (int s0 = 0; s0 < n_seq && seq < 0; s0 += kWave) {
             const int s = s0 + lane;
             const int c = s < n_seq ? max(ctx_lens[s], 0) : 0;
@@ -123,6 +158,7 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
                 ctx_raw = __builtin_amdgcn_readlane(c, src);
             }
             base += __builtin_amdgcn_readlane(inc, kWave - 1);
+        }
         }
         if (seq < 0) return;                                // beyond the last item (whole workgroup)
     } else {

@@ -281,6 +281,10 @@ def main() -> int:
                "sample": r["sample"] + "; decode (LUT gather) + fp32 torch.mv, pack excluded",
                "pack_us": round(r["pack_s"] * 1e6, 1), "decode_us": round(r["decode_s"] * 1e6, 1),
                "compute_us": round(r["compute_s"] * 1e6, 1), "cpu_count": r["cpu_count"]}
+        # second half of the metric: decode + fp32 SDPA per head (B4 H16 d=64 L=8192, E5M2), two heads timed
+        ra = cpu_baseline.attention_baseline(64, 8192, 64, "E5M2", sample_heads=2, repeats=3)
+        cpu["flash_attn_e5m2_b4h16_d64_L8192_us"] = round(ra["total_s"] * 1e6, 1)
+        cpu["flash_attn_sample"] = ra["sample"] + "; decode (LUT gather) + fp32 SDPA per head, median of 3"
 
     line = {
         "metric": "packed-FP8 GEMV us (16384^2, E4M3, FP32 accumulate)",

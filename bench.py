@@ -168,6 +168,12 @@ def main() -> int:
                              args.warmup, sync)
             extra[f"dot_{mode.lower()}_2p24_us"] = round(us, 2)
             extra[f"dot_{mode.lower()}_2p24_GBps"] = round((2 * n + 4) / us / 1e3, 1)
+        # dot, n = 16384 (one workgroup, one launch: latency bound)
+        xs_s = [x[:4096] for x in xs]
+        for mode in ("E4M3", "E5M2"):
+            us = gpu_time_us(lambda i: feather.dot(xs_s[(2 * i) % 64], xs_s[(2 * i + 1) % 64], mode=mode),
+                             args.steps, args.warmup, sync)
+            extra[f"dot_{mode.lower()}_16384_us"] = round(us, 2)
         # pack throughput (2 B in + 1 B out per element)
         src = randn(8192, 16384).half()
         for mode in ("E5M2", "E4M3"):

@@ -97,7 +97,9 @@ __global__ __launch_bounds__(kDotThreads) void dot_kernel(const uint32_t *__rest
         float t = 0.f;
 #pragma unroll
         for (int w = 0; w < kDotThreads / kWave; w++) t += wave_part[w];
-        reinterpret_cast<float *>(scratch + 16)[blockIdx.x] = t;
+        // a single workgroup holds the whole sum: no second kernel (the launch is half of a short dot's time)
+        if (gridDim.x == 1) out[0] = t;
+        else reinterpret_cast<float *>(scratch + 16)[blockIdx.x] = t;
     }
 }
 
@@ -143,7 +145,7 @@ static int launch_dot(const void *x1, const void *x2, void *out, void *scratch, 
         hipLaunchKernelGGL((dot_kernel<KIND, false>), dim3((unsigned)blocks), dim3(kDotThreads), 0, s,
                            (const uint32_t *)x1, (const uint32_t *)x2, (float *)out, (uint32_t *)scratch, n_words);
     int rc = check_launch(what);
-    if (rc != FEATHER_OK) return rc;
+    if (rc != FEATHER_OK || blocks == 1) return rc;
     hipLaunchKernelGGL(dot_finish_kernel, dim3(1), dim3(kFinishThreads), 0, s, (const uint32_t *)scratch, (float *)out,
                        (int)blocks);
     return check_launch(what);

@@ -4,7 +4,8 @@
 // reads 128-bit chunks of both vectors, decodes in registers and accumulates
 // with v_dot2_f32_f16.  The reduction is deterministic: every workgroup writes
 // one partial to scratch and a second one-wave kernel adds the partials in
-// index order.  (A single-kernel "last workgroup finishes" scheme needs
+// index order; an input that a single workgroup covers (up to 4096 words) is
+// finished by that workgroup and needs no second launch.  (A single-kernel "last workgroup finishes" scheme needs
 // device-scope release/acquire around the arrival counter, which on this
 // multi-XCD part costs an L2 write-back/invalidate per workgroup and measured
 // ~45 us for 2^24 elements; the second launch costs a few us.  The same scheme

@@ -51,7 +51,8 @@ __device__ __forceinline__ half8_t bg_dec8(uint32_t w0, uint32_t w1) {
 // of the same indices, and the epilogue writes pack(fp16(silu(gate) * up)) as FP8 words to
 // `packed` ([nvec, inter / 4]) instead of fp32 sums to `out` (one K slice only).
 // KG: K groups per workgroup (1 or 2); every slice must hold a multiple of KG chunks.
-template <int MODE, int NB, bool SWIGLU, int KG>
+// ROT: rotated K walk (long walks only, see below).
+template <int MODE, int NB, bool SWIGLU, int KG, bool ROT = false>
 __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uint8_t *__restrict__ w,
                                                                  const uint8_t *__restrict__ x,
                                                                  float *__restrict__ out, int M, int K, int nvec,
@@ -95,8 +96,8 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
         for (int i = 0; i < NB; i++) xr[i] = xok[i] ? *reinterpret_cast<const u32x4 *>(xp[i] + col) : u32x4{0, 0, 0, 0};
     };
     // One chunk: vectors' chunk -> LDS, (the caller's prefetch goes here), barrier, MFMAs.
-    auto stage_x = [&](int c, const u32x4 (&xr)[NB]) {
-        _Float16 *buf = xs + (((c - c_begin) / KG) & 1) * (16 * NB * kBgPitch);
+    auto stage_x = [&](int it, const u32x4 (&xr)[NB]) {
+        _Float16 *buf = xs + ((it / KG) & 1) * (16 * NB * kBgPitch);
 #pragma unroll
         for (int i = 0; i < NB; i++) {
             *reinterpret_cast<half8_t *>(buf + xdst[i]) = bg_dec8<MODE>(xr[i].x, xr[i].y);
@@ -117,14 +118,25 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
         }
     };
     if (c_begin >= c_end) return;                  // cannot happen: the launcher creates no empty slice
-    issue(c_begin + grp, wa, xa);
+    // ROT: every row tile starts its K walk at another chunk and wraps around.  With a common start all
+    // workgroups read the same column offsets at the same time, addresses that differ by multiples of
+    // the row pitch and fall on few memory channels (16384 x 16384, 32 vectors, E5M2: 72 -> 56 us).
+    // Walks of a few chunks gain nothing from it and keep the plain order.
+    const int n_it = c_end - c_begin;              // a multiple of KG
+    const int rot = ROT ? (int)((blockIdx.x * 7u) % (unsigned)(n_it / KG)) * KG : 0;
+    auto chunk_of = [&](int it) {
+        if constexpr (!ROT) return c_begin + it;
+        int t = it + rot;
+        return c_begin + (t >= n_it ? t - n_it : t);
+    };
+    issue(chunk_of(grp), wa, xa);
     // Every chunk but the last prefetches its successor unconditionally, so the number of loads
     // in flight is known at compile time and the wait for chunk c leaves chunk c + 1 outstanding
     // (a prefetch inside an `if` makes the compiler wait for everything).
-    for (int c = c_begin + grp; c < c_end - KG; c += KG) {
-        const _Float16 *buf = stage_x(c, xa);
+    for (int it = grp; it < n_it - KG; it += KG) {
+        const _Float16 *buf = stage_x(it, xa);
         u32x4 wn[4], xn[NB];
-        issue(c + KG, wn, xn);
+        issue(chunk_of(it + KG), wn, xn);
         __syncthreads();
         mac(buf, wa);
 #pragma unroll
@@ -133,7 +145,7 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
         for (int i = 0; i < NB; i++) xa[i] = xn[i];
     }
     {
-        const _Float16 *buf = stage_x(c_end - KG + grp, xa);
+        const _Float16 *buf = stage_x(n_it - KG + grp, xa);
         __syncthreads();
         mac(buf, wa);
     }
@@ -195,13 +207,13 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
     }
 }
 
-template <int MODE, int NB, bool SWIGLU, int KG>
+template <int MODE, int NB, bool SWIGLU, int KG, bool ROT = false>
 static void bg_launch_kg(const void *w, const void *x, float *out, int M, int K, int nvec, int splits, int cps,
                          int64_t part_stride, uint32_t *packed, hipStream_t s) {
     const size_t lds = (size_t)KG * 2 * 16 * NB * kBgPitch * sizeof(_Float16);
     static unsigned long long lds_raised = 0;      // per instantiation, one bit per device
-    (void)raise_lds_limit(reinterpret_cast<const void *>(&gemv_batched_kernel<MODE, NB, SWIGLU, KG>), lds, lds_raised);
-    hipLaunchKernelGGL((gemv_batched_kernel<MODE, NB, SWIGLU, KG>),
+    (void)raise_lds_limit(reinterpret_cast<const void *>(&gemv_batched_kernel<MODE, NB, SWIGLU, KG, ROT>), lds, lds_raised);
+    hipLaunchKernelGGL((gemv_batched_kernel<MODE, NB, SWIGLU, KG, ROT>),
                        dim3((unsigned)((M + kBgRows - 1) / kBgRows), (unsigned)splits), dim3(kBgThreads * KG), lds, s,
                        (const uint8_t *)w, (const uint8_t *)x, out, M, K, nvec, cps, part_stride, packed);
 }
@@ -215,7 +227,15 @@ static void bg_launch(const void *w, const void *x, float *out, int M, int K, in
                       int64_t part_stride, uint32_t *packed, hipStream_t s) {
     const int last = K / kBgChunk - (splits - 1) * cps;   // chunks of the last slice
     const int64_t groups = (int64_t)((M + kBgRows - 1) / kBgRows) * splits;
-    if (cps >= 4 && cps % 2 == 0 && last % 2 == 0 && (groups <= 256 || cps >= 16))
+    const bool two = cps >= 4 && cps % 2 == 0 && last % 2 == 0 && (groups <= 256 || cps >= 16);
+    if constexpr (!SWIGLU) {
+        if (cps >= 32 && last >= 32) {             // long K walk: rotated start per row tile
+            if (two) bg_launch_kg<MODE, NB, false, 2, true>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);
+            else bg_launch_kg<MODE, NB, false, 1, true>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);
+            return;
+        }
+    }
+    if (two)
         bg_launch_kg<MODE, NB, SWIGLU, 2>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);
     else
         bg_launch_kg<MODE, NB, SWIGLU, 1>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);

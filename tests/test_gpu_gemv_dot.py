@@ -140,7 +140,9 @@ def test_gemv_rejects_bad_shapes(dev):
 
 @pytest.mark.parametrize("mode", ["E4M3", "E5M2"])
 @pytest.mark.parametrize("M,K,nvec", [(2048, 2048, 32), (256, 5632, 32), (50, 512, 5), (33, 1024, 64), (16, 100, 3), (130, 768, 17),
-                                      (6, 256, 1), (4100, 2048, 48), (130, 4096, 17), (70, 1536, 9)])
+                                      (6, 256, 1), (4100, 2048, 48), (130, 4096, 17), (70, 1536, 9),
+                                      # K walks of >= 32 chunks start at a rotated chunk per row tile (one and two K groups)
+                                      (200, 8192, 32), (70, 8448, 5), (130, 16384, 17), (1100, 8192, 64)])
 def test_gemv_batched_vs_oracle(dev, orc, mode, M, K, nvec):
     from feather_amd.routines.gemv import gemv_fp8_batched_acc_fp32_gpu
     rng = np.random.default_rng(M + K + nvec)

@@ -151,6 +151,14 @@ def main() -> int:
         extra["gemv_e5m2_16384_us"] = round(us, 2)
         extra["gemv_e5m2_16384_GBps"] = round(gemv_bytes / us / 1e3, 1)
         extra["gemv_e5m2_16384_hbm_frac"] = round(gemv_bytes / us / 1e3 / HBM_PEAK_GBS, 4)
+        # batched GEMV: the same rotating E5M2 matrices against 32 vectors (weights streamed once per batch)
+        from feather_amd.routines.gemv import gemv_fp8_batched_acc_fp32_gpu
+        xb = feather.pack_fp8_tensor(randn(32, K).half(), mode="E5M2")
+        us = gpu_time_us(lambda i: gemv_fp8_batched_acc_fp32_gpu(mats["E5M2"][i % NBUF], xb, (M, K), 32, "E5M2"),
+                         50, 10, sync)
+        extra["gemv_batched_e5m2_16384_x32_us"] = round(us, 2)
+        extra["gemv_batched_e5m2_16384_x32_GBps"] = round((M * K + 32 * K + 4 * 32 * M) / us / 1e3, 1)
+        del xb
         # config 0: 8192 x 8192 E5M2 (views into the 16384^2 buffers: 4 distinct 64 MiB matrices each)
         M0 = K0 = 8192
         sub = [b[i * (M0 * K0 // 4):(i + 1) * (M0 * K0 // 4)] for b in mats["E5M2"] for i in range(4)]

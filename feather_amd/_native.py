@@ -46,6 +46,8 @@ SIGNATURES = {
     "feather_paged_attn_scratch_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "feather_paged_attn_fp8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                       _i32, _f32, _vp]),
+    "feather_paged_attn_fp8_static": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                             _i32, _f32, _vp]),
     "feather_decode_step_scratch_bytes": (_i64, [_vp, _i64, _i64]),
     "feather_decode_step": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp]),
 }

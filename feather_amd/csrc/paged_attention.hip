@@ -24,6 +24,8 @@
 // without the second launch but was slower: write-through stores, the ticket and
 // the read-back are three memory-side round trips in a row, +7 us per call
 // against ~4 us for the merge kernel.)
+#include <mutex>
+
 #include "internal.h"
 #include "common.h"
 
@@ -554,4 +556,59 @@ extern "C" int feather_paged_attn_fp8(const void *q, const void *k_cache, const 
                   FEATHER_EINVAL, "%s: misaligned pointer", me);
     return paged_attn_launch(q, k_cache, v_cache, block_tables, ctx_lens, (float *)out_f32, nullptr, nullptr, scratch, n_seq,
                              n_q_heads, n_kv_heads, d, block_size, max_blocks, max_ctx, mode, scale, (hipStream_t)stream);
+}
+
+// ---- the same attention for callers that cannot allocate -------------------------------------
+// The split partials live in a file-scope device array instead of a caller-supplied buffer.  Every
+// device that loads the library holds its own copy of the array at its own address, which
+// hipGetSymbolAddress returns for the current device; host code only ever uses that address (the
+// array's name is a host-side handle, not device memory).
+namespace feather {
+
+static __device__ __align__(256) unsigned char g_pa_static_scratch[FEATHER_PAGED_ATTN_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static void *g_pa_static_ptr[kMaxDevices];   // device address of the array, per device; set once
+static std::mutex g_pa_static_mutex;
+
+static int pa_static_scratch(void **out, const char *me) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    FEATHER_CHECK(e == hipSuccess, FEATHER_ELAUNCH, "%s: hipGetDevice: %s", me, hipGetErrorString(e));
+    FEATHER_CHECK(dev >= 0 && dev < kMaxDevices, FEATHER_EINVAL, "%s: device index %d outside 0..%d", me, dev,
+                  kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(g_pa_static_mutex);
+    if (!g_pa_static_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_pa_static_scratch));
+        FEATHER_CHECK(e == hipSuccess && p, FEATHER_ELAUNCH, "%s: hipGetSymbolAddress: %s", me, hipGetErrorString(e));
+        g_pa_static_ptr[dev] = p;
+    }
+    *out = g_pa_static_ptr[dev];
+    return FEATHER_OK;
+}
+
+}  // namespace feather
+
+extern "C" int feather_paged_attn_fp8_static(const void *q, const void *k_cache, const void *v_cache,
+                                             const void *block_tables, const void *ctx_lens, void *out_f32,
+                                             int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads, int64_t d,
+                                             int64_t block_size, int64_t max_blocks, int64_t max_ctx, int mode,
+                                             float scale, void *stream) {
+    const char *me = "feather_paged_attn_fp8_static";
+    const int64_t need = feather_paged_attn_scratch_bytes(n_seq, n_q_heads, d, max_ctx);
+    FEATHER_CHECK(need <= (int64_t)FEATHER_PAGED_ATTN_STATIC_SCRATCH_BYTES, FEATHER_ESHAPE,
+                  "%s: the split partials of this problem need %lld bytes, the built-in buffer holds %lld "
+                  "(n_seq * n_q_heads * ceil(max_ctx / 512) * (d + 2) * 4); use feather_paged_attn_fp8 with a "
+                  "caller-owned scratch",
+                  me, (long long)need, (long long)FEATHER_PAGED_ATTN_STATIC_SCRATCH_BYTES);
+    void *scratch = nullptr;
+    if (n_seq > 0) {
+        int rc = pa_static_scratch(&scratch, me);
+        if (rc != FEATHER_OK) return rc;
+    }
+    // nothing in the buffer has to start at zero: the merge reads only the partials of splits that
+    // hold tokens, and the split kernel of the same call writes exactly those
+    return feather_paged_attn_fp8(q, k_cache, v_cache, block_tables, ctx_lens, out_f32, scratch, n_seq, n_q_heads,
+                                  n_kv_heads, d, block_size, max_blocks, max_ctx, mode, scale, stream);
 }

@@ -170,6 +170,21 @@ int feather_paged_attn_fp8(const void *q, const void *k_cache, const void *v_cac
                            int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks, int64_t max_ctx,
                            int mode, float scale, void *stream);
 
+/* feather_paged_attn_fp8 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.
+ * Same arguments without `scratch`: the split partials go to a buffer of
+ * FEATHER_PAGED_ATTN_STATIC_SCRATCH_BYTES that is part of the library's device image (every GPU the
+ * library runs on holds it until the process ends).  A problem whose
+ * feather_paged_attn_scratch_bytes() exceeds that size is rejected with FEATHER_ESHAPE.  The call
+ * allocates and frees nothing.  All calls on one GPU share the buffer: calls that overlap on one
+ * GPU (different streams, or threads) race; calls on one stream are ordered and safe.  Nothing in
+ * the buffer needs clearing between calls.  Results are bit-identical to feather_paged_attn_fp8. */
+#define FEATHER_PAGED_ATTN_STATIC_SCRATCH_BYTES (4 << 20)
+int feather_paged_attn_fp8_static(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,
+                                  const void *ctx_lens, void *out_f32, int64_t n_seq, int64_t n_q_heads,
+                                  int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
+                                  int64_t max_ctx, int mode, float scale, void *stream);
+
 /* ---- decode step of a Llama-shaped model on packed weights (no reference counterpart) ----
  *
  * The reference has no model code; this entry point runs one token step for a batch with

@@ -3,7 +3,12 @@ TEST INFRASTRUCTURE ONLY.  The step is build-defined (the reference has no model
 this file fixes its meaning: float32 element-wise math, every GEMV operand rounded
 fp32 -> fp16 -> FP8 (RNE) and decoded with the kernel decode, GEMV sums in float64.
 Parity status: the pieces (quant, rmsnorm, rope, online_attention) are pinned by closed forms
-in tests/test_oracle.py; the composition has no external reference: parity unpinned."""
+in tests/test_oracle.py.  The composition (layer order, residual placement, q/k/v row split of the
+fused projection, grouped-query head mapping, cache position and block addressing, gate/up split) is
+pinned there too: with ``mode=None`` (no quantiser, float caches) decode_step_ref must equal an
+independent float64 Llama step assembled from torch library routines on separate q/k/v/o/gate/up/down
+weights, and that check is shown to fail for swapped k/v rows, a shifted head mapping and a dropped
+residual."""
 from __future__ import annotations
 
 import numpy as np
@@ -11,8 +16,10 @@ import numpy as np
 from . import decode_np, pack_fp8
 
 
-def quant(x: np.ndarray, mode: str) -> np.ndarray:
-    """fp32 array -> decoded values after fp16 + FP8 rounding (same shape, float64)."""
+def quant(x: np.ndarray, mode) -> np.ndarray:
+    """fp32 array -> decoded values after fp16 + FP8 rounding (same shape, float64); mode None: no rounding."""
+    if mode is None:
+        return np.asarray(x, dtype=np.float64)
     with np.errstate(over="ignore"):
         words = pack_fp8(x.astype(np.float32).astype(np.float16), mode)
     return decode_np(words, mode)[: x.size].reshape(x.shape)
@@ -86,9 +93,14 @@ def online_attention(dots: np.ndarray, V: np.ndarray, scale: float, chunk: int =
     return (num / float(den)).astype(np.float32)
 
 
-def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables, ctx_lens, mode: str):
+def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables, ctx_lens, mode):
     """weights: fp16 numpy arrays under the names of PackedDecoder; k_caches / v_caches: per-layer
-    uint32 arrays [n_blocks, n_kv, block_size, d/4], updated in place.  Returns logits [B, vocab] float32."""
+    uint32 arrays [n_blocks, n_kv, block_size, d/4], updated in place.  Returns logits [B, vocab] float32.
+    mode None runs the same composition without any FP8 rounding on float caches
+    [n_blocks, n_kv, block_size, d] (used to pin the composition against library routines)."""
+    store = (lambda a: quant_codes(a, mode)) if mode is not None else (lambda a: np.asarray(a, dtype=np.float32))
+    load = (lambda w_, n_, d_: decode_np(w_, mode).reshape(n_, d_)) if mode is not None else \
+        (lambda w_, n_, d_: np.asarray(w_, dtype=np.float64).reshape(n_, d_))
     H, nq, nkv, d, I = cfg.hidden, cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.inter
     B = len(tokens)
     Wq = lambda a: quant(np.asarray(a, dtype=np.float32), mode)                  # packed weight values
@@ -108,8 +120,8 @@ def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables
             v = heads[nq + nkv:]
             blk, slot = int(block_tables[b][pos // cfg.block_size]), pos % cfg.block_size
             for kvh in range(nkv):
-                k_caches[l][blk, kvh, slot] = quant_codes(k[kvh], mode)
-                v_caches[l][blk, kvh, slot] = quant_codes(v[kvh], mode)
+                k_caches[l][blk, kvh, slot] = store(k[kvh])
+                v_caches[l][blk, kvh, slot] = store(v[kvh])
             qd = quant(q, mode)
             n = pos + 1
             for hq in range(nq):
@@ -117,8 +129,8 @@ def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables
                 rows = [(int(block_tables[b][t // cfg.block_size]), t % cfg.block_size) for t in range(n)]
                 Kw = np.stack([k_caches[l][bb, kvh, ss] for bb, ss in rows])
                 Vw = np.stack([v_caches[l][bb, kvh, ss] for bb, ss in rows])
-                Kd = decode_np(Kw, mode).reshape(n, d)
-                Vd = decode_np(Vw, mode).reshape(n, d)
+                Kd = load(Kw, n, d)
+                Vd = load(Vw, n, d)
                 attn[b, hq * d:(hq + 1) * d] = online_attention(Kd @ qd[hq], Vd, float(scale))
         o = (quant(attn, mode) @ Wq(g("wo")).T).astype(np.float32)
         h = h + o

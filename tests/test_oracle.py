@@ -466,3 +466,97 @@ def test_paged_cache_write_oracle_places_rows(orc):
             assert (vc[bt[s, pos // bs], :, pos % bs] == v[:, cu[s] + i]).all()
             written += 1
     assert written == 5 + 6 and (kc.reshape(-1, dw).any(axis=1).sum() == written * n_kv)
+
+
+# ---------------------------------------------------------------- decode step: the composition
+
+def _llama_step_f64(cfg, w, k_cache, v_cache, tokens, bt, ctx, bug=None):
+    """One Llama decode step in float64 from torch library routines only, on SEPARATE q/k/v/o/gate/up/down
+    weights and float caches [n_blocks, n_kv, block_size, d] per layer (updated in place).  Written
+    independently of oracle/decode_ref.py: complex-multiplication RoPE, F.rms_norm, F.silu,
+    F.scaled_dot_product_attention over the gathered cache with repeated KV heads.  `bug` plants one
+    composition mistake, to show that the comparison would catch it."""
+    F = torch.nn.functional
+    t = lambda a: torch.as_tensor(np.asarray(a, dtype=np.float64))
+    H, nq, nkv, d, bs = cfg.hidden, cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size
+    inv = cfg.rope_theta ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)          # theta^(-2j/d)
+
+    def rot(x, pos):                                   # rotate-half: (x_j, x_{j+d/2}) is one complex number
+        z = torch.complex(x[..., : d // 2], x[..., d // 2:]) * torch.polar(torch.ones_like(inv), pos * inv)
+        return torch.cat([z.real, z.imag], dim=-1)
+
+    h = t(w["embed"])[torch.as_tensor(np.asarray(tokens, dtype=np.int64))]
+    for l in range(cfg.n_layers):
+        g = lambda n: t(w[f"{l}.{n}"])
+        x = F.rms_norm(h, (H,), g("norm_attn"), cfg.rms_eps)
+        q, k, v = x @ g("wq").T, x @ g("wk").T, x @ g("wv").T
+        if bug == "swap_kv":
+            k, v = v, k
+        att = torch.zeros_like(q)
+        for b in range(len(tokens)):
+            pos = int(ctx[b]) + (1 if bug == "position" else 0)
+            qb = rot(q[b].view(nq, d), pos)
+            kb = rot(k[b].view(nkv, d), pos)
+            blk, slot = int(bt[b][int(ctx[b]) // bs]), int(ctx[b]) % bs
+            k_cache[l][blk, :, slot] = kb
+            v_cache[l][blk, :, slot] = v[b].view(nkv, d)
+            n = int(ctx[b]) + 1
+            blocks = torch.as_tensor(np.asarray(bt[b][: (n + bs - 1) // bs], dtype=np.int64))
+            K = k_cache[l][blocks].permute(1, 0, 2, 3).reshape(nkv, -1, d)[:, :n]      # [nkv, n, d]
+            V = v_cache[l][blocks].permute(1, 0, 2, 3).reshape(nkv, -1, d)[:, :n]
+            if bug == "head_map":                      # query head h -> KV head h % nkv instead of h // group
+                K, V = K.repeat(nq // nkv, 1, 1), V.repeat(nq // nkv, 1, 1)
+            else:
+                K, V = K.repeat_interleave(nq // nkv, dim=0), V.repeat_interleave(nq // nkv, dim=0)
+            att[b] = F.scaled_dot_product_attention(qb[:, None, :], K, V).reshape(-1)
+        o = att @ g("wo").T
+        h = o if bug == "residual" else h + o
+        x = F.rms_norm(h, (H,), g("norm_mlp"), cfg.rms_eps)
+        gate, up = x @ g("w_gate").T, x @ g("w_up").T
+        if bug == "gate_up":
+            gate, up = up, gate
+        h = h + (F.silu(gate) * up) @ g("w_down").T
+    return (F.rms_norm(h, (H,), t(w["norm_final"]), cfg.rms_eps) @ t(w["lm_head"]).T).numpy()
+
+
+def test_decode_step_ref_composition_matches_library_llama_step(orc):
+    """Pins the composition of decode_step_ref (which the GPU decode step is checked against): without
+    the quantiser it is an ordinary Llama decode step, so it must agree with a float64 step built from
+    torch library routines; only the fp16 rounding of P inside online_attention separates them
+    (<= 2^-11 relative per term).  Planted composition mistakes must break the agreement."""
+    import types
+    from oracle import decode_ref
+    cfg = types.SimpleNamespace(n_layers=2, hidden=128, n_q_heads=4, n_kv_heads=2, head_dim=32, inter=192, vocab=50,
+                                block_size=4, rms_eps=1e-5, rope_theta=10000.0)
+    rng = np.random.default_rng(12)
+    rn = lambda *s: rng.standard_normal(s).astype(np.float32)
+    H, nq, nkv, d, I = cfg.hidden, cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.inter
+    w = {"embed": rn(cfg.vocab, H), "norm_final": 1 + 0.1 * rn(H), "lm_head": rn(cfg.vocab, H) / np.sqrt(H)}
+    for l in range(cfg.n_layers):
+        w.update({f"{l}.wq": rn(nq * d, H) / np.sqrt(H), f"{l}.wk": rn(nkv * d, H) / np.sqrt(H),
+                  f"{l}.wv": rn(nkv * d, H) / np.sqrt(H), f"{l}.wo": rn(H, nq * d) / np.sqrt(H),
+                  f"{l}.w_gate": rn(I, H) / np.sqrt(H), f"{l}.w_up": rn(I, H) / np.sqrt(H),
+                  f"{l}.w_down": rn(H, I) / np.sqrt(I), f"{l}.norm_attn": 1 + 0.1 * rn(H), f"{l}.norm_mlp": 1 + 0.1 * rn(H)})
+    B, max_blocks = 3, 5
+    n_blocks = B * max_blocks + 1
+    bt = rng.permutation(n_blocks)[: B * max_blocks].reshape(B, max_blocks).astype(np.int32)
+    ctx = np.array([0, 7, 18], dtype=np.int32)                 # empty cache, mid-block, first slot of a later block... (18 % 4 = 2)
+    tokens = np.array([3, 11, 42], dtype=np.int32)
+    caches = [rn(n_blocks, nkv, cfg.block_size, d) for _ in range(2 * cfg.n_layers)]
+    fresh = lambda as_torch: [torch.as_tensor(c.astype(np.float64)) if as_torch else c.copy() for c in caches]
+
+    kc, vc = fresh(False)[: cfg.n_layers], fresh(False)[cfg.n_layers:]
+    got = decode_ref.decode_step_ref(cfg, w, kc, vc, tokens, bt, ctx, None)
+    tk, tv = fresh(True)[: cfg.n_layers], fresh(True)[cfg.n_layers:]
+    want = _llama_step_f64(cfg, w, tk, tv, tokens, bt, ctx)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() / scale < 5e-4
+    for l in range(cfg.n_layers):                               # the appended rows, and nothing else, changed
+        tol = 1e-5 if l == 0 else 1e-3                          # layer 0 has no attention (fp16 P) upstream
+        assert np.abs(kc[l] - tk[l].numpy()).max() < tol and np.abs(vc[l] - tv[l].numpy()).max() < tol
+        changed = np.argwhere(np.any(kc[l] != caches[l], axis=-1))
+        assert sorted(map(tuple, changed)) == sorted((int(bt[b][ctx[b] // 4]), kv, int(ctx[b] % 4)) for b in range(B) for kv in range(nkv))
+    for bug in ("swap_kv", "head_map", "residual", "gate_up", "position"):
+        tk, tv = fresh(True)[: cfg.n_layers], fresh(True)[cfg.n_layers:]
+        wrong = _llama_step_f64(cfg, w, tk, tv, tokens, bt, ctx, bug=bug)
+        assert np.abs(got - wrong).max() / scale > 2e-2, f"planted mistake '{bug}' would go unnoticed"

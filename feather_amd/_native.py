@@ -30,11 +30,13 @@ SIGNATURES = {
     "feather_version": (_i32, []),
     "feather_last_error": (ctypes.c_char_p, []),
     "feather_pack_fp8": (_i32, [_vp, _vp, _i64, _i32, _i32, _vp]),
+    "feather_quant_pack_f32": (_i32, [_vp, _vp, _i64, _i32, _vp]),
     "feather_unpack_fp8": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp]),
     "feather_pack_fp16": (_i32, [_vp, _vp, _i64, _vp]),
     "feather_unpack_fp16": (_i32, [_vp, _vp, _i64, _vp]),
     "feather_gemv_fp8": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp]),
     "feather_gemv_fp8_batched": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp]),
+    "feather_gemv_fp8_batched_swiglu": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp]),
     "feather_dot_scratch_bytes": (_i64, []),
     "feather_dot_fp8": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _vp]),
     "feather_dot_fp16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _vp]),
@@ -42,14 +44,17 @@ SIGNATURES = {
     "feather_flash_attn_fp8_varlen": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _f32,
                                              _i32, _vp]),
     "feather_paged_cache_write": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
-                                         _i32, _vp]),
+                                         _i64, _i32, _vp]),
     "feather_paged_attn_scratch_bytes": (_i64, [_i64, _i64, _i64, _i64]),
-    "feather_paged_attn_fp8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
-                                      _i32, _f32, _vp]),
-    "feather_paged_attn_fp8_static": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
-                                             _i32, _f32, _vp]),
+    "feather_paged_attn_fp8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                      _i64, _i32, _f32, _vp]),
+    "feather_paged_attn_fp8_static": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
+                                             _i64, _i64, _i32, _f32, _vp]),
     "feather_decode_step_scratch_bytes": (_i64, [_vp, _i64, _i64]),
-    "feather_decode_step": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp]),
+    "feather_decode_step": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "feather_add_rmsnorm_pack": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _vp]),
+    "feather_rope_append": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
+                                   _i64, _i64, _f32, _i32, _vp]),
 }
 
 
@@ -64,7 +69,7 @@ class Decoder(ctypes.Structure):
     _fields_ = [("n_layers", ctypes.c_int32), ("hidden", ctypes.c_int32), ("n_q_heads", ctypes.c_int32),
                 ("n_kv_heads", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("inter", ctypes.c_int32),
                 ("vocab", ctypes.c_int32), ("block_size", ctypes.c_int32), ("max_blocks", ctypes.c_int32),
-                ("mode", ctypes.c_int32), ("rms_eps", _f32), ("rope_theta", _f32),
+                ("n_blocks", ctypes.c_int32), ("mode", ctypes.c_int32), ("rms_eps", _f32), ("rope_theta", _f32),
                 ("layers", ctypes.POINTER(DecoderLayer)), ("embed_f16", _vp), ("norm_final", _vp),
                 ("w_lm_head", _vp)]
 

@@ -617,6 +617,8 @@ extern "C" int feather_flash_attn_fp8(const void *q, const void *k, const void *
     FEATHER_CHECK(tail == FEATHER_TAIL_MASK || tail == FEATHER_TAIL_REFERENCE, FEATHER_EINVAL,
                   "feather_flash_attn_fp8: bad tail flag %d", tail);
     FEATHER_CHECK(n_heads >= 0 && L >= 0 && d > 0, FEATHER_EINVAL, "feather_flash_attn_fp8: negative shape");
+    FEATHER_CHECK(scale > 0.f, FEATHER_EINVAL,
+                  "feather_flash_attn_fp8: scale must be positive (the running maximum is kept on raw scores)");
     FEATHER_CHECK(kv_group >= 1 && n_heads % kv_group == 0, FEATHER_ESHAPE,
                   "feather_flash_attn_fp8: n_heads=%lld is not a multiple of kv_group=%lld", (long long)n_heads,
                   (long long)kv_group);
@@ -640,6 +642,7 @@ extern "C" int feather_flash_attn_fp8_varlen(const void *q, const void *k, const
     FEATHER_CHECK(n_heads >= 0 && n_seq >= 0 && max_seqlen >= 0 && total_rows >= 0 && d > 0, FEATHER_EINVAL,
                   "%s: negative shape", me);
     FEATHER_CHECK(causal == 0 || causal == 1, FEATHER_EINVAL, "%s: causal must be 0 or 1", me);
+    FEATHER_CHECK(scale > 0.f, FEATHER_EINVAL, "%s: scale must be positive (the running maximum is kept on raw scores)", me);
     FEATHER_CHECK(kv_group >= 1 && n_heads % kv_group == 0, FEATHER_ESHAPE,
                   "%s: n_heads=%lld is not a multiple of kv_group=%lld", me, (long long)n_heads, (long long)kv_group);
     FEATHER_CHECK(max_seqlen <= total_rows && total_rows < (1ll << 30), FEATHER_ESHAPE,

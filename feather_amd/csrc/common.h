@@ -175,7 +175,11 @@ __device__ __forceinline__ uint32_t enc(uint32_t h) {
 // pack_fp8_tensor applied to an fp32 producer
 template <int MODE>
 __device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d) {
-    // fp32 -> fp16 (round to nearest even) -> FP8 code (round to nearest even)
+    // fp32 -> fp16 (round to nearest even) -> FP8 code (round to nearest even).
+    // The values are pinned in registers first: when an argument is a product, the compiler otherwise
+    // folds multiply and conversion into v_fma_mixlo_f16 x, y, +0, and (-0) + (+0) = +0 loses the sign of
+    // a zero product (code 0x00 instead of 0x80).
+    asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
     uint32_t h0 = __builtin_bit_cast(uint16_t, (_Float16)a), h1 = __builtin_bit_cast(uint16_t, (_Float16)b);
     uint32_t h2 = __builtin_bit_cast(uint16_t, (_Float16)c), h3 = __builtin_bit_cast(uint16_t, (_Float16)d);
     if constexpr (MODE == FEATHER_E5M2)

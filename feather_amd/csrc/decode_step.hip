@@ -74,7 +74,7 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_pack_kernel(float *__rest
                                                                      int64_t part_stride,
                                                                      const float *__restrict__ w,
                                                                      uint32_t *__restrict__ xq, int hidden,
-                                                                     float eps) {
+                                                                     float eps, float *__restrict__ y_f32) {
     __shared__ float red[THREADS / kWave];
     const int b = blockIdx.x;
     float4 *hr = reinterpret_cast<float4 *>(h + (int64_t)b * hidden);
@@ -133,13 +133,17 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_pack_kernel(float *__rest
 #pragma unroll
     for (int it = 0; it < kKeep; it++) {
         const int i = threadIdx.x + it * THREADS;
-        if (i < n4)
-            xq[(int64_t)b * n4 + i] = quant4<MODE>(x[it].x * r * g[it].x, x[it].y * r * g[it].y, x[it].z * r * g[it].z,
-                                                  x[it].w * r * g[it].w);
+        if (i < n4) {
+            const float4 y = make_float4(x[it].x * r * g[it].x, x[it].y * r * g[it].y, x[it].z * r * g[it].z, x[it].w * r * g[it].w);
+            xq[(int64_t)b * n4 + i] = quant4<MODE>(y.x, y.y, y.z, y.w);
+            if (y_f32) reinterpret_cast<float4 *>(y_f32)[(int64_t)b * n4 + i] = y;   // the values the codes were rounded from
+        }
     }
     for (int i = threadIdx.x + kKeep * THREADS; i < n4; i += THREADS) {
         float4 y = hr[i], gg = wr[i];
-        xq[(int64_t)b * n4 + i] = quant4<MODE>(y.x * r * gg.x, y.y * r * gg.y, y.z * r * gg.z, y.w * r * gg.w);
+        y = make_float4(y.x * r * gg.x, y.y * r * gg.y, y.z * r * gg.z, y.w * r * gg.w);
+        xq[(int64_t)b * n4 + i] = quant4<MODE>(y.x, y.y, y.z, y.w);
+        if (y_f32) reinterpret_cast<float4 *>(y_f32)[(int64_t)b * n4 + i] = y;
     }
 }
 
@@ -151,11 +155,11 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_pack_kernel(float *__rest
 // and two idle slots: 2.1 us from entry to the sums; see the launcher of the decode step).
 template <int MODE>
 static void launch_norm(int batch, hipStream_t s, float *h, const float *delta, int n_part, int64_t part_stride,
-                        const void *w, uint32_t *xq, int hidden, float eps) {
+                        const void *w, uint32_t *xq, int hidden, float eps, float *y_f32 = nullptr) {
     const int n4 = hidden / 4;
     auto go = [&](auto kern, int threads) {
         hipLaunchKernelGGL(kern, dim3(batch), dim3(threads), 0, s, h, delta, n_part, part_stride, (const float *)w, xq,
-                           hidden, eps);
+                           hidden, eps, y_f32);
     };
     if (n4 <= 256) go(add_rmsnorm_pack_kernel<MODE, 1, 256>, 256);
     else if (n4 <= 512) go(add_rmsnorm_pack_kernel<MODE, 1, 512>, 512);
@@ -184,6 +188,9 @@ __global__ __launch_bounds__(kDsThreads) void swiglu_pack_kernel(const float *__
 // qkv [B, (n_q + 2 n_kv) * d] fp32 -> RoPE on q and k (rotate-half convention: element j pairs
 // with j + d/2, angle pos * theta^(-2j/d)), q packed to qp [B, n_q, d/4], k and v encoded and
 // written into the paged cache at position pos = ctx_lens[b]; ctx_after[b] = pos + 1.
+// A position outside [0, max_blocks * block_size) or a block id outside [0, n_blocks) is never
+// written: the token is dropped, ctx_after[b] is the old length (clamped into the table) and
+// status[b] says why (1: no room / bad position, 2: bad block id; 0: appended).
 constexpr int kRopeThreads = 64;
 // sin and cos of a non-negative angle below ~1e5 rad to ~1e-7 absolute: three-constant Cody-Waite reduction
 // by pi/2 with fused multiply-adds, then the single-precision minimax polynomials on [-pi/4, pi/4].  The
@@ -212,7 +219,9 @@ __global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *
                                                                 float log2_theta, uint32_t *__restrict__ qp,
                                                                 uint32_t *__restrict__ k_cache,
                                                                 uint32_t *__restrict__ v_cache,
-                                                                int32_t *__restrict__ ctx_after) {
+                                                                int32_t *__restrict__ ctx_after, int n_blocks,
+                                                                int32_t *__restrict__ status,
+                                                                float *__restrict__ rot_f32) {
     const int b = blockIdx.x;
     const int dw = d / 4, half_w = d / 8;            // words per head, words per rotation half
     const int heads = n_q + 2 * n_kv;
@@ -232,9 +241,17 @@ __global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *
         pl[u] = *reinterpret_cast<const float4 *>(x + 4 * t + off);            // elements 4t .. 4t+3
         ph[u] = *reinterpret_cast<const float4 *>(x + d / 2 + 4 * t + off);    // their partners
     }
-    const int pos = min(pos_raw, max_blocks * block_size - 1);
-    if (threadIdx.x == 0 && blockIdx.y == 0) ctx_after[b] = pos + 1;
-    const int64_t slot = ((int64_t)block_tables[(int64_t)b * max_blocks + pos / block_size] * n_kv) * block_size;
+    const int cap = max_blocks * block_size;
+    const bool pos_ok = pos_raw >= 0 && pos_raw < cap;
+    const int pos = pos_ok ? pos_raw : 0;            // in range for the table lookup; nothing is written if !pos_ok
+    const int blk = block_tables[(int64_t)b * max_blocks + pos / block_size];
+    const bool blk_ok = (unsigned)blk < (unsigned)n_blocks;
+    const bool append = pos_ok && blk_ok;
+    if (threadIdx.x == 0 && blockIdx.y == 0) {
+        ctx_after[b] = append ? pos + 1 : min(max(pos_raw, 0), cap);
+        if (status) status[b] = pos_ok ? (blk_ok ? 0 : 2) : 1;
+    }
+    const int64_t slot = ((int64_t)(blk_ok ? blk : 0) * n_kv) * block_size;
     float4 lo = pl[0], hi = ph[0];                   // slices are added in index order
 #pragma unroll
     for (int u = 1; u < G; u++)
@@ -273,10 +290,16 @@ __global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *
             hi = make_float4(hi4[0], hi4[1], hi4[2], hi4[3]);
         }
         const uint32_t wlo = quant4<MODE>(lo.x, lo.y, lo.z, lo.w), whi = quant4<MODE>(hi.x, hi.y, hi.z, hi.w);
+        if (rot_f32) {                               // the values the codes were rounded from
+            float *r = rot_f32 + ((int64_t)b * heads + head) * d;
+            *reinterpret_cast<float4 *>(r + 4 * t) = lo;
+            *reinterpret_cast<float4 *>(r + d / 2 + 4 * t) = hi;
+        }
         uint32_t *dst;
         if (head < n_q) {
             dst = qp + ((int64_t)b * n_q + head) * dw;
         } else {
+            if (!append) return;
             const int kvh = head < n_q + n_kv ? head - n_q : head - n_q - n_kv;
             uint32_t *cache = head < n_q + n_kv ? k_cache : v_cache;
             dst = cache + ((slot + (int64_t)kvh * block_size) + pos % block_size) * dw;
@@ -328,7 +351,8 @@ static StepPlan plan_step(const feather_decoder_t *dec, int64_t batch) {
 
 template <int MODE>
 static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const int32_t *block_tables,
-                    const int32_t *ctx_lens, int batch, int max_ctx, void *scratch, float *logits, hipStream_t s) {
+                    const int32_t *ctx_lens, int batch, int max_ctx, void *scratch, float *logits, int32_t *status,
+                    hipStream_t s) {
     const int H = dec->hidden, nq = dec->n_q_heads, nkv = dec->n_kv_heads, d = dec->head_dim, I = dec->inter;
     const StepPlan P = plan_step(dec, batch);
     const int qkv_rows = (int)P.qkv_rows;
@@ -378,16 +402,17 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
         hipLaunchKernelGGL((rope_append_kernel<MODE>),
                            dim3(batch, ((nq + 2 * nkv) * (d / 8) + kRopeThreads - 1) / kRopeThreads), dim3(kRopeThreads), 0, s, qkv, ctx_lens,
                            block_tables, (int64_t)batch * qkv_rows, P.s_qkv, nq, nkv, d, dec->block_size, dec->max_blocks,
-                           log2_theta, qp, (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, ctx_after);
+                           log2_theta, qp, (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, ctx_after, dec->n_blocks,
+                           l == 0 ? status : nullptr, (float *)nullptr);
         DS_CHECK(check_launch("feather_decode_step (rope)"));
         // attention writes its output already rounded to FP8 and packed (the operand of W_o)
         DS_CHECK(paged_attn_launch(qp, L.k_cache, L.v_cache, block_tables, ctx_after, nullptr, xq, nullptr, pa_scratch, batch, nq,
-                                   nkv, d, dec->block_size, dec->max_blocks, max_ctx, MODE, scale, s));
+                                   nkv, d, dec->block_size, dec->max_blocks, dec->n_blocks, max_ctx, MODE, scale, s));
         DS_CHECK(gemv(L.w_o, delta, H, nq * d, P.s_o));
         launch_norm<MODE>(batch, s, h, delta, P.s_o, hs, L.norm_mlp, xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
         if (P.fused_mlp) {
-            DS_CHECK(gemv_batched_swiglu_launch(L.w_gate_up, xq, act, I, H, batch, MODE, s));
+            DS_CHECK(gemv_batched_swiglu_launch(L.w_gate_up, xq, act, nullptr, I, H, batch, MODE, s));
         } else {
             DS_CHECK(gemv(L.w_gate_up, gu, 2 * I, H, P.s_gu));
             int64_t items = (int64_t)batch * I / 4;
@@ -421,7 +446,8 @@ static int check_decoder(const feather_decoder_t *dec, int64_t batch, int64_t ma
     FEATHER_CHECK(dec->mode == FEATHER_E5M2 || dec->mode == FEATHER_E4M3, FEATHER_EMODE, "%s: mode %d not supported", me,
                   dec->mode);
     FEATHER_CHECK(dec->n_layers >= 0 && dec->hidden > 0 && dec->n_q_heads > 0 && dec->n_kv_heads > 0 &&
-                      dec->head_dim > 0 && dec->inter > 0 && dec->vocab > 0 && dec->block_size > 0 && dec->max_blocks > 0,
+                      dec->head_dim > 0 && dec->inter > 0 && dec->vocab > 0 && dec->block_size > 0 && dec->max_blocks > 0 &&
+                      dec->n_blocks > 0,
                   FEATHER_EINVAL, "%s: bad configuration", me);
     FEATHER_CHECK(dec->hidden == dec->n_q_heads * dec->head_dim, FEATHER_ESHAPE, "%s: hidden != n_q_heads * head_dim", me);
     FEATHER_CHECK(dec->head_dim == 64 || dec->head_dim == 128 || dec->head_dim == 256, FEATHER_ESHAPE,
@@ -443,7 +469,7 @@ extern "C" int64_t feather_decode_step_scratch_bytes(const feather_decoder_t *de
 
 extern "C" int feather_decode_step(const feather_decoder_t *dec, const void *token_ids, const void *block_tables,
                                    const void *ctx_lens, int64_t batch, int64_t max_ctx, void *scratch,
-                                   void *logits_f32, void *stream) {
+                                   void *logits_f32, void *seq_status, void *stream) {
     const char *me = "feather_decode_step";
     int rc = check_decoder(dec, batch, max_ctx, me);
     if (rc != FEATHER_OK) return rc;
@@ -455,11 +481,74 @@ extern "C" int feather_decode_step(const feather_decoder_t *dec, const void *tok
         FEATHER_CHECK(L.w_qkv && L.w_o && L.w_gate_up && L.w_down && L.norm_attn && L.norm_mlp && L.k_cache && L.v_cache,
                       FEATHER_EINVAL, "%s: null pointer in layer %d", me, l);
     }
-    FEATHER_CHECK(aligned(scratch, 256) && aligned(logits_f32, 16), FEATHER_EINVAL, "%s: misaligned scratch/logits", me);
+    FEATHER_CHECK(aligned(scratch, 256) && aligned(logits_f32, 16) && aligned(seq_status, 4), FEATHER_EINVAL,
+                  "%s: misaligned scratch/logits/status", me);
     hipStream_t s = (hipStream_t)stream;
     if (dec->mode == FEATHER_E5M2)
         return run_step<FEATHER_E5M2>(dec, (const int32_t *)token_ids, (const int32_t *)block_tables,
-                                      (const int32_t *)ctx_lens, (int)batch, (int)max_ctx, scratch, (float *)logits_f32, s);
+                                      (const int32_t *)ctx_lens, (int)batch, (int)max_ctx, scratch, (float *)logits_f32,
+                                      (int32_t *)seq_status, s);
     return run_step<FEATHER_E4M3>(dec, (const int32_t *)token_ids, (const int32_t *)block_tables,
-                                  (const int32_t *)ctx_lens, (int)batch, (int)max_ctx, scratch, (float *)logits_f32, s);
+                                  (const int32_t *)ctx_lens, (int)batch, (int)max_ctx, scratch, (float *)logits_f32,
+                                      (int32_t *)seq_status, s);
+}
+
+// ---- the fused producers of the step as entry points of their own -------------------------------
+
+extern "C" int feather_add_rmsnorm_pack(void *h_f32, const void *delta_f32, int64_t n_part, int64_t part_stride,
+                                        const void *gain_f32, void *xq_u32, void *y_f32, int64_t batch, int64_t hidden,
+                                        float eps, int mode, void *stream) {
+    const char *me = "feather_add_rmsnorm_pack";
+    FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE, "%s: mode %d not supported", me, mode);
+    FEATHER_CHECK(batch >= 0 && batch < (1ll << 31) && hidden > 0 && hidden < (1ll << 31), FEATHER_EINVAL, "%s: bad shape", me);
+    FEATHER_CHECK(hidden % 4 == 0, FEATHER_ESHAPE, "%s: hidden=%lld is not a multiple of 4", me, (long long)hidden);
+    FEATHER_CHECK(!delta_f32 || (n_part >= 1 && n_part <= 64 && part_stride >= 0 && part_stride % 4 == 0), FEATHER_EINVAL,
+                  "%s: n_part must be in [1, 64] and part_stride a non-negative multiple of 4", me);
+    FEATHER_CHECK(eps >= 0.f, FEATHER_EINVAL, "%s: negative eps", me);
+    if (batch == 0) return FEATHER_OK;
+    FEATHER_CHECK(h_f32 && gain_f32 && xq_u32, FEATHER_EINVAL, "%s: null pointer", me);
+    FEATHER_CHECK(aligned(h_f32, 16) && aligned(delta_f32, 16) && aligned(gain_f32, 16) && aligned(xq_u32, 4) && aligned(y_f32, 16),
+                  FEATHER_EINVAL, "%s: misaligned pointer", me);
+    hipStream_t s = (hipStream_t)stream;
+    if (mode == FEATHER_E5M2)
+        launch_norm<FEATHER_E5M2>((int)batch, s, (float *)h_f32, (const float *)delta_f32, (int)n_part, part_stride, gain_f32,
+                                  (uint32_t *)xq_u32, (int)hidden, eps, (float *)y_f32);
+    else
+        launch_norm<FEATHER_E4M3>((int)batch, s, (float *)h_f32, (const float *)delta_f32, (int)n_part, part_stride, gain_f32,
+                                  (uint32_t *)xq_u32, (int)hidden, eps, (float *)y_f32);
+    return check_launch(me);
+}
+
+extern "C" int feather_rope_append(const void *qkv_f32, int64_t n_part, int64_t part_stride, const void *ctx_lens,
+                                   const void *block_tables, void *q_packed, void *k_cache, void *v_cache, void *ctx_after,
+                                   void *seq_status, void *rot_f32, int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
+                                   int64_t d, int64_t block_size, int64_t max_blocks, int64_t n_blocks, float rope_theta,
+                                   int mode, void *stream) {
+    const char *me = "feather_rope_append";
+    FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE, "%s: mode %d not supported", me, mode);
+    FEATHER_CHECK(batch >= 0 && batch < 65536 && n_q_heads > 0 && n_kv_heads > 0 && block_size > 0 && max_blocks > 0 &&
+                      n_blocks > 0 && n_blocks < (1ll << 31) && max_blocks * block_size < (1ll << 31),
+                  FEATHER_EINVAL, "%s: bad shape", me);
+    FEATHER_CHECK(d > 0 && d % 8 == 0 && d <= 1024, FEATHER_ESHAPE, "%s: head dim %lld is not a multiple of 8", me, (long long)d);
+    FEATHER_CHECK(n_part >= 1 && n_part <= 64 && part_stride >= 0 && part_stride % 4 == 0, FEATHER_EINVAL,
+                  "%s: n_part must be in [1, 64] and part_stride a non-negative multiple of 4", me);
+    FEATHER_CHECK(rope_theta > 0.f, FEATHER_EINVAL, "%s: rope_theta must be positive", me);
+    if (batch == 0) return FEATHER_OK;
+    FEATHER_CHECK(qkv_f32 && ctx_lens && block_tables && q_packed && k_cache && v_cache && ctx_after, FEATHER_EINVAL,
+                  "%s: null pointer", me);
+    FEATHER_CHECK(aligned(qkv_f32, 16) && aligned(ctx_lens, 4) && aligned(block_tables, 4) && aligned(q_packed, 4) &&
+                      aligned(k_cache, 4) && aligned(v_cache, 4) && aligned(ctx_after, 4) && aligned(seq_status, 4) &&
+                      aligned(rot_f32, 16),
+                  FEATHER_EINVAL, "%s: misaligned pointer", me);
+    const int heads = (int)(n_q_heads + 2 * n_kv_heads);
+    const dim3 grid((unsigned)batch, (unsigned)((heads * (d / 8) + kRopeThreads - 1) / kRopeThreads));
+#define FEATHER_ROPE(MM)                                                                                                \
+    hipLaunchKernelGGL((rope_append_kernel<MM>), grid, dim3(kRopeThreads), 0, (hipStream_t)stream, (const float *)qkv_f32, \
+                       (const int32_t *)ctx_lens, (const int32_t *)block_tables, part_stride, (int)n_part, (int)n_q_heads, \
+                       (int)n_kv_heads, (int)d, (int)block_size, (int)max_blocks, log2f(rope_theta), (uint32_t *)q_packed, \
+                       (uint32_t *)k_cache, (uint32_t *)v_cache, (int32_t *)ctx_after, (int)n_blocks, (int32_t *)seq_status, \
+                       (float *)rot_f32)
+    if (mode == FEATHER_E5M2) FEATHER_ROPE(FEATHER_E5M2); else FEATHER_ROPE(FEATHER_E4M3);
+#undef FEATHER_ROPE
+    return check_launch(me);
 }

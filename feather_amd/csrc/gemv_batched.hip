@@ -57,7 +57,8 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
                                                                  const uint8_t *__restrict__ x,
                                                                  float *__restrict__ out, int M, int K, int nvec,
                                                                  int cps, int64_t part_stride,
-                                                                 uint32_t *__restrict__ packed) {
+                                                                 uint32_t *__restrict__ packed,
+                                                                 float *__restrict__ act_f32) {
     extern __shared__ __attribute__((aligned(16))) _Float16 xs_all[];   // [KG][2][16 * NB][kBgPitch]
     const int lane = threadIdx.x & 63;
     const int grp = KG == 1 ? 0 : wave_id() / 4, wave = KG == 1 ? wave_id() : wave_id() % 4;
@@ -183,8 +184,9 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
                 auto f = [](float a, float b) {
                     return a * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * a)) * b;
                 };
-                packed[(int64_t)vec * (inter / 4) + g / 4] =
-                    quant4<MODE>(f(acc[nb][0], u[0]), f(acc[nb][1], u[1]), f(acc[nb][2], u[2]), f(acc[nb][3], u[3]));
+                const float4_t a = float4_t{f(acc[nb][0], u[0]), f(acc[nb][1], u[1]), f(acc[nb][2], u[2]), f(acc[nb][3], u[3])};
+                packed[(int64_t)vec * (inter / 4) + g / 4] = quant4<MODE>(a[0], a[1], a[2], a[3]);
+                if (act_f32) *reinterpret_cast<float4_t *>(act_f32 + (int64_t)vec * inter + g) = a;   // the values the codes were rounded from
             }
         }
         return;
@@ -209,13 +211,13 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
 
 template <int MODE, int NB, bool SWIGLU, int KG, bool ROT = false>
 static void bg_launch_kg(const void *w, const void *x, float *out, int M, int K, int nvec, int splits, int cps,
-                         int64_t part_stride, uint32_t *packed, hipStream_t s) {
+                         int64_t part_stride, uint32_t *packed, float *act_f32, hipStream_t s) {
     const size_t lds = (size_t)KG * 2 * 16 * NB * kBgPitch * sizeof(_Float16);
     static unsigned long long lds_raised = 0;      // per instantiation, one bit per device
     (void)raise_lds_limit(reinterpret_cast<const void *>(&gemv_batched_kernel<MODE, NB, SWIGLU, KG, ROT>), lds, lds_raised);
     hipLaunchKernelGGL((gemv_batched_kernel<MODE, NB, SWIGLU, KG, ROT>),
                        dim3((unsigned)((M + kBgRows - 1) / kBgRows), (unsigned)splits), dim3(kBgThreads * KG), lds, s,
-                       (const uint8_t *)w, (const uint8_t *)x, out, M, K, nvec, cps, part_stride, packed);
+                       (const uint8_t *)w, (const uint8_t *)x, out, M, K, nvec, cps, part_stride, packed, act_f32);
 }
 
 // Two K groups per workgroup when every slice (the last one too) gives each group at least two chunks
@@ -224,21 +226,21 @@ static void bg_launch_kg(const void *w, const void *x, float *out, int M, int K,
 // 8 chunks) 18.1 -> 18.7 us; four groups (1024 threads) were slower than two on every shape tried.
 template <int MODE, int NB, bool SWIGLU>
 static void bg_launch(const void *w, const void *x, float *out, int M, int K, int nvec, int splits, int cps,
-                      int64_t part_stride, uint32_t *packed, hipStream_t s) {
+                      int64_t part_stride, uint32_t *packed, float *act_f32, hipStream_t s) {
     const int last = K / kBgChunk - (splits - 1) * cps;   // chunks of the last slice
     const int64_t groups = (int64_t)((M + kBgRows - 1) / kBgRows) * splits;
     const bool two = cps >= 4 && cps % 2 == 0 && last % 2 == 0 && (groups <= 256 || cps >= 16);
     if constexpr (!SWIGLU) {
         if (cps >= 32 && last >= 32) {             // long K walk: rotated start per row tile
-            if (two) bg_launch_kg<MODE, NB, false, 2, true>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);
-            else bg_launch_kg<MODE, NB, false, 1, true>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);
+            if (two) bg_launch_kg<MODE, NB, false, 2, true>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, act_f32, s);
+            else bg_launch_kg<MODE, NB, false, 1, true>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, act_f32, s);
             return;
         }
     }
     if (two)
-        bg_launch_kg<MODE, NB, SWIGLU, 2>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);
+        bg_launch_kg<MODE, NB, SWIGLU, 2>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, act_f32, s);
     else
-        bg_launch_kg<MODE, NB, SWIGLU, 1>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, s);
+        bg_launch_kg<MODE, NB, SWIGLU, 1>(w, x, out, M, K, nvec, splits, cps, part_stride, packed, act_f32, s);
 }
 
 int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M, int64_t K, int64_t nvec, int mode,
@@ -249,7 +251,7 @@ int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M,
     splits = (n_chunks + cps - 1) / cps;           // no empty slice
     if (splits_out) *splits_out = splits;
     const int nb = (int)((nvec + 15) / 16);
-#define FEATHER_BG(MM, NBB) bg_launch<MM, NBB, false>(w, x, out_f32, (int)M, (int)K, (int)nvec, splits, cps, part_stride, nullptr, stream)
+#define FEATHER_BG(MM, NBB) bg_launch<MM, NBB, false>(w, x, out_f32, (int)M, (int)K, (int)nvec, splits, cps, part_stride, nullptr, nullptr, stream)
     if (mode == FEATHER_E5M2) {
         switch (nb) { case 1: FEATHER_BG(FEATHER_E5M2, 1); break; case 2: FEATHER_BG(FEATHER_E5M2, 2); break;
                       case 3: FEATHER_BG(FEATHER_E5M2, 3); break; default: FEATHER_BG(FEATHER_E5M2, 4); }
@@ -263,12 +265,12 @@ int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M,
 
 // act = pack(fp16(silu(W_gate x) * (W_up x))) with w = [gate rows; up rows] ([2 * inter, K]); the
 // GEMV and the activation in one kernel, no fp32 round trip.  Needs K % 256 == 0, inter % 4 == 0.
-int gemv_batched_swiglu_launch(const void *w, const void *x, uint32_t *act_packed, int64_t inter, int64_t K,
-                               int64_t nvec, int mode, hipStream_t stream) {
+int gemv_batched_swiglu_launch(const void *w, const void *x, uint32_t *act_packed, float *act_f32, int64_t inter,
+                               int64_t K, int64_t nvec, int mode, hipStream_t stream) {
     const int n_chunks = (int)(K / kBgChunk);
     const int nb = (int)((nvec + 15) / 16);
 #define FEATHER_BG(MM, NBB) \
-    bg_launch<MM, NBB, true>(w, x, nullptr, (int)(2 * inter), (int)K, (int)nvec, 1, n_chunks, 0, act_packed, stream)
+    bg_launch<MM, NBB, true>(w, x, nullptr, (int)(2 * inter), (int)K, (int)nvec, 1, n_chunks, 0, act_packed, act_f32, stream)
     if (mode == FEATHER_E5M2) {
         switch (nb) { case 1: FEATHER_BG(FEATHER_E5M2, 1); break; case 2: FEATHER_BG(FEATHER_E5M2, 2); break;
                       case 3: FEATHER_BG(FEATHER_E5M2, 3); break; default: FEATHER_BG(FEATHER_E5M2, 4); }
@@ -304,4 +306,22 @@ extern "C" int feather_gemv_fp8_batched(const void *w, const void *x, void *out_
         return FEATHER_OK;
     }
     return gemv_batched_launch(w, x, (float *)out_f32, M, K, nvec, mode, 1, 0, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int feather_gemv_fp8_batched_swiglu(const void *w_gate_up, const void *x, void *act_packed, void *act_f32,
+                                               int64_t inter, int64_t K, int64_t nvec, int mode, void *stream) {
+    const char *me = "feather_gemv_fp8_batched_swiglu";
+    FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE, "%s: mode %d not supported", me, mode);
+    FEATHER_CHECK(inter >= 0 && K >= 0, FEATHER_EINVAL, "%s: negative shape", me);
+    FEATHER_CHECK(nvec >= 1 && nvec <= 64, FEATHER_ESHAPE, "%s: nvec=%lld outside [1, 64]", me, (long long)nvec);
+    FEATHER_CHECK(K > 0 && K % kBgChunk == 0, FEATHER_ESHAPE, "%s: K=%lld is not a positive multiple of %d", me, (long long)K,
+                  kBgChunk);
+    FEATHER_CHECK(inter % 4 == 0, FEATHER_ESHAPE, "%s: inter=%lld is not a multiple of 4", me, (long long)inter);
+    FEATHER_CHECK(2 * inter < (1ll << 31) && K < (1ll << 31), FEATHER_ESHAPE, "%s: shape too large", me);
+    if (inter == 0) return FEATHER_OK;
+    FEATHER_CHECK(w_gate_up && x && act_packed, FEATHER_EINVAL, "%s: null pointer", me);
+    FEATHER_CHECK(aligned(w_gate_up, 16) && aligned(x, 16) && aligned(act_packed, 4) && aligned(act_f32, 16), FEATHER_EINVAL,
+                  "%s: misaligned pointer", me);
+    return gemv_batched_swiglu_launch(w_gate_up, x, (uint32_t *)act_packed, (float *)act_f32, inter, K, nvec, mode,
+                                      (hipStream_t)stream);
 }

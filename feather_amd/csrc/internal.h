@@ -13,7 +13,7 @@ namespace feather {
 int paged_attn_launch(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,
                       const void *ctx_lens, float *out_f32, uint32_t *out_packed, _Float16 *out_q16, void *scratch, int64_t n_seq,
                       int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
-                      int64_t max_ctx, int mode, float scale, hipStream_t stream);
+                      int64_t n_blocks, int64_t max_ctx, int mode, float scale, hipStream_t stream);
 
 // Batched GEMV with the K range cut into `splits` slices: slice s writes its partial sums to
 // out_f32 + s * part_stride ([nvec, M] each); the consumer adds the slices in index order.
@@ -24,8 +24,9 @@ int gemv_batched_launch(const void *w, const void *x, float *out_f32, int64_t M,
 
 // As gemv_batched_launch for w = [gate rows; up rows] ([2 * inter, K]) with the SwiGLU activation
 // and the FP8 quantisation fused: act_packed [nvec, inter / 4] words.  Needs K % 256 == 0,
-// inter % 4 == 0, 16-byte aligned w and x.
-int gemv_batched_swiglu_launch(const void *w, const void *x, uint32_t *act_packed, int64_t inter, int64_t K,
-                               int64_t nvec, int mode, hipStream_t stream);
+// inter % 4 == 0, 16-byte aligned w and x.  act_f32 (optional, [nvec, inter]) receives the fp32 values the
+// codes were rounded from.
+int gemv_batched_swiglu_launch(const void *w, const void *x, uint32_t *act_packed, float *act_f32, int64_t inter,
+                               int64_t K, int64_t nvec, int mode, hipStream_t stream);
 
 }  // namespace feather

@@ -14,7 +14,7 @@ __global__ __launch_bounds__(256) void paged_cache_write_kernel(
     const void *__restrict__ k_src, const void *__restrict__ v_src, uint32_t *__restrict__ k_cache,
     uint32_t *__restrict__ v_cache, const int32_t *__restrict__ block_tables, const int32_t *__restrict__ cu_seqlens,
     const int32_t *__restrict__ start_pos, int n_seq, int total_rows, int n_kv_heads, int units, int block_size,
-    int max_blocks) {
+    int max_blocks, int n_blocks) {
     const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;      // 16-code unit
     if (u >= (int64_t)n_kv_heads * total_rows * units) return;
     const int c = (int)(u % units);
@@ -29,6 +29,7 @@ __global__ __launch_bounds__(256) void paged_cache_write_kernel(
     const int pos = (start_pos ? start_pos[lo] : 0) + t - cu_seqlens[lo];
     if (pos < 0 || pos >= max_blocks * block_size) return;          // no entry in the block table: dropped
     const int blk = block_tables[(int64_t)lo * max_blocks + pos / block_size];
+    if ((unsigned)blk >= (unsigned)n_blocks) return;                // padding or a bad entry: dropped, never written
     const int64_t dst = ((((int64_t)blk * n_kv_heads + h) * block_size + pos % block_size) * units + c) * 4;
     const int64_t src = ((int64_t)h * total_rows + t) * units + c;  // in 16-code units
 #pragma unroll
@@ -57,12 +58,14 @@ using namespace feather;
 extern "C" int feather_paged_cache_write(const void *k_src, const void *v_src, int src_f16, void *k_cache, void *v_cache,
                                          const void *block_tables, const void *cu_seqlens, const void *start_pos,
                                          int64_t n_seq, int64_t total_rows, int64_t n_kv_heads, int64_t d,
-                                         int64_t block_size, int64_t max_blocks, int mode, void *stream) {
+                                         int64_t block_size, int64_t max_blocks, int64_t n_blocks, int mode,
+                                         void *stream) {
     const char *me = "feather_paged_cache_write";
     FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE, "%s: mode %d not supported", me, mode);
     FEATHER_CHECK(src_f16 == 0 || src_f16 == 1, FEATHER_EINVAL, "%s: src_f16 must be 0 or 1", me);
-    FEATHER_CHECK(n_seq >= 0 && total_rows >= 0 && n_kv_heads >= 0 && block_size > 0 && max_blocks >= 0, FEATHER_EINVAL,
-                  "%s: bad shape", me);
+    FEATHER_CHECK(n_seq >= 0 && total_rows >= 0 && n_kv_heads >= 0 && block_size > 0 && max_blocks >= 0 && n_blocks >= 0,
+                  FEATHER_EINVAL, "%s: bad shape", me);
+    FEATHER_CHECK(n_blocks < (1ll << 31), FEATHER_ESHAPE, "%s: n_blocks too large", me);
     FEATHER_CHECK(d > 0 && d % 16 == 0, FEATHER_ESHAPE, "%s: head dim %lld is not a multiple of 16", me, (long long)d);
     FEATHER_CHECK(total_rows < (1ll << 31) && max_blocks * block_size < (1ll << 31), FEATHER_ESHAPE, "%s: shape too large", me);
     if (n_seq == 0 || total_rows == 0 || n_kv_heads == 0) return FEATHER_OK;
@@ -76,7 +79,8 @@ extern "C" int feather_paged_cache_write(const void *k_src, const void *v_src, i
     hipLaunchKernelGGL((paged_cache_write_kernel<MM, FF>), dim3((unsigned)((units + 255) / 256)), dim3(256), 0,       \
                        (hipStream_t)stream, k_src, v_src, (uint32_t *)k_cache, (uint32_t *)v_cache,                   \
                        (const int32_t *)block_tables, (const int32_t *)cu_seqlens, (const int32_t *)start_pos,        \
-                       (int)n_seq, (int)total_rows, (int)n_kv_heads, (int)(d / 16), (int)block_size, (int)max_blocks)
+                       (int)n_seq, (int)total_rows, (int)n_kv_heads, (int)(d / 16), (int)block_size, (int)max_blocks,    \
+                       (int)n_blocks)
     if (mode == FEATHER_E5M2) { if (src_f16) FEATHER_CW(FEATHER_E5M2, true); else FEATHER_CW(FEATHER_E5M2, false); }
     else { if (src_f16) FEATHER_CW(FEATHER_E4M3, true); else FEATHER_CW(FEATHER_E4M3, false); }
 #undef FEATHER_CW

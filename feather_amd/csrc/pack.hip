@@ -93,6 +93,56 @@ static int launch_pack(const void *src, void *dst, int64_t n, hipStream_t s) {
     return check_launch("feather_pack_fp8");
 }
 
+// ---------------------------------------------------------------- fp32 -> packed fp8
+
+// The rounding chain of an fp32 producer that feeds a packed GEMV: fp32 -> fp16 (RNE) -> FP8 code
+// (RNE), four codes per word (quant4).  Thread t converts elements [16t, 16t+16) from four 128-bit
+// loads to one 128-bit store; the tail is handled one word per thread with zero padding.
+template <int MODE, bool ALIGNED>
+__global__ __launch_bounds__(256) void quant_pack_f32_kernel(const float *__restrict__ src, uint32_t *__restrict__ dst,
+                                                            int64_t n, int64_t n16) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t g = t; g < n16; g += stride) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float4_t v;
+            if constexpr (ALIGNED) v = __builtin_nontemporal_load(reinterpret_cast<const float4_t *>(src) + 4 * g + i);
+            else v = float4_t{src[16 * g + 4 * i], src[16 * g + 4 * i + 1], src[16 * g + 4 * i + 2], src[16 * g + 4 * i + 3]};
+            w[i] = quant4<MODE>(v[0], v[1], v[2], v[3]);
+        }
+        if constexpr (ALIGNED) {
+            store_nt128(reinterpret_cast<u32x4 *>(dst) + g, u32x4{w[0], w[1], w[2], w[3]});
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[4 * g + i] = w[i];
+        }
+    }
+    const int64_t first = 16 * n16, tail_words = (n - first + 3) / 4;
+    if (t < tail_words) {
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] = first + 4 * t + i < n ? src[first + 4 * t + i] : 0.f;
+        dst[first / 4 + t] = quant4<MODE>(v[0], v[1], v[2], v[3]);
+    }
+}
+
+template <int MODE>
+static int launch_quant_pack(const void *src, void *dst, int64_t n, hipStream_t s) {
+    const int64_t n16 = n / 16;
+    const bool al = aligned(src, 16) && aligned(dst, 16);
+    int64_t blocks = ((n16 > 4 ? n16 : 4) + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    if (al)
+        hipLaunchKernelGGL((quant_pack_f32_kernel<MODE, true>), dim3((unsigned)blocks), dim3(256), 0, s, (const float *)src,
+                           (uint32_t *)dst, n, n16);
+    else
+        hipLaunchKernelGGL((quant_pack_f32_kernel<MODE, false>), dim3((unsigned)blocks), dim3(256), 0, s, (const float *)src,
+                           (uint32_t *)dst, n, n16);
+    return check_launch("feather_quant_pack_f32");
+}
+
 // ---------------------------------------------------------------- unpack fp8
 
 template <int MODE, int SEM>
@@ -227,6 +277,17 @@ extern "C" int feather_pack_fp8(const void *src_f16, void *dst_u32, int64_t n, i
     if (rounding == FEATHER_ROUND_TRUNC) return launch_pack<FEATHER_E5M2, FEATHER_ROUND_TRUNC>(src_f16, dst_u32, n, s);
     if (mode == FEATHER_E5M2) return launch_pack<FEATHER_E5M2, FEATHER_ROUND_RNE>(src_f16, dst_u32, n, s);
     return launch_pack<FEATHER_E4M3, FEATHER_ROUND_RNE>(src_f16, dst_u32, n, s);
+}
+
+extern "C" int feather_quant_pack_f32(const void *src_f32, void *dst_u32, int64_t n, int mode, void *stream) {
+    FEATHER_CHECK(n >= 0, FEATHER_EINVAL, "feather_quant_pack_f32: negative n");
+    FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE,
+                  "feather_quant_pack_f32: mode %d not supported", mode);
+    if (n == 0) return FEATHER_OK;
+    FEATHER_CHECK(src_f32 && dst_u32, FEATHER_EINVAL, "feather_quant_pack_f32: null pointer");
+    FEATHER_CHECK(aligned(src_f32, 4) && aligned(dst_u32, 4), FEATHER_EINVAL, "feather_quant_pack_f32: misaligned pointer");
+    if (mode == FEATHER_E5M2) return launch_quant_pack<FEATHER_E5M2>(src_f32, dst_u32, n, (hipStream_t)stream);
+    return launch_quant_pack<FEATHER_E4M3>(src_f32, dst_u32, n, (hipStream_t)stream);
 }
 
 extern "C" int feather_unpack_fp8(const void *src_u32, void *dst, int64_t n_words, int mode, int semantics,

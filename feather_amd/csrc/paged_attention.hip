@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     const int32_t *__restrict__ ctx_lens, const int32_t *__restrict__ block_tables, const uint32_t *__restrict__ q,
     const uint32_t *__restrict__ k_cache, const uint32_t *__restrict__ v_cache, int n_q_heads, int n_kv_heads,
     int block_size, int max_blocks, int n_splits, int max_ctx, float scale_log2e, float *__restrict__ scratch,
-    float *__restrict__ out_f32, uint32_t *__restrict__ out_packed, _Float16 *__restrict__ out_q16) {
+    float *__restrict__ out_f32, uint32_t *__restrict__ out_packed, _Float16 *__restrict__ out_q16, uint32_t max_blk) {
     const int bs_shift = FAST ? __builtin_ctz((unsigned)block_size) : 0;
     constexpr int DW = D / 4;       // words per token row
     constexpr int RB = D / 64;      // 16-word row blocks of V per token
@@ -243,7 +243,11 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     // stay in registers).  Rows past the context read the fallback block (valid memory) and are
     // masked later.
     // row index inside the cache in 32 bits (a cache of 2^31 rows of d codes is >= 128 GB)
-    auto row_base = [&](int blk, int tok) { return (int64_t)(uint32_t)((blk * n_kv_heads + kvh) * block_size + slot_of(tok)); };
+    // block ids come from the caller's table: an id outside the cache (padding, -1) is clamped to the last block,
+    // so that a bad table gives a wrong result for that sequence and never an access outside the cache
+    auto row_base = [&](int blk, int tok) {
+        return (int64_t)(uint32_t)((min((uint32_t)blk, max_blk) * n_kv_heads + kvh) * block_size + slot_of(tok));
+    };
     auto load_step = [&](Step &S, int t0) {
         const bool full = t0 + kStepTok <= ctx;   // wave-uniform: every token of the step exists
 #pragma unroll
@@ -475,7 +479,7 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const float *__re
 template <int D, int MODE>
 static int launch_paged(const void *q, const void *kc, const void *vc, const void *bt, const void *cl, float *out_f32,
                         uint32_t *out_packed, _Float16 *out_q16, void *scratch, int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads,
-                        int64_t block_size, int64_t max_blocks, int64_t max_ctx, float scale, hipStream_t s) {
+                        int64_t block_size, int64_t max_blocks, int64_t n_blocks, int64_t max_ctx, float scale, hipStream_t s) {
     int n_splits = (int)((max_ctx + kSplit - 1) / kSplit);
     if (n_splits < 1) n_splits = 1;
     int64_t blocks = n_seq * n_kv_heads * n_splits;
@@ -488,12 +492,12 @@ static int launch_paged(const void *q, const void *kc, const void *vc, const voi
         hipLaunchKernelGGL((paged_attn_split_kernel<D, MODE, true>), dim3((unsigned)blocks), dim3(kPaThreads), 0, s,
                            (const int32_t *)cl, (const int32_t *)bt, (const uint32_t *)q, (const uint32_t *)kc,
                            (const uint32_t *)vc, (int)n_q_heads, (int)n_kv_heads, (int)block_size, (int)max_blocks, n_splits,
-                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16);
+                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16, (uint32_t)(n_blocks - 1));
     else
         hipLaunchKernelGGL((paged_attn_split_kernel<D, MODE, false>), dim3((unsigned)blocks), dim3(kPaThreads), 0, s,
                            (const int32_t *)cl, (const int32_t *)bt, (const uint32_t *)q, (const uint32_t *)kc,
                            (const uint32_t *)vc, (int)n_q_heads, (int)n_kv_heads, (int)block_size, (int)max_blocks, n_splits,
-                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16);
+                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16, (uint32_t)(n_blocks - 1));
     int rc = check_launch("feather_paged_attn_fp8");
     if (rc != FEATHER_OK || n_splits == 1) return rc;
     int64_t threads = n_seq * n_q_heads * (D / 4);
@@ -507,10 +511,10 @@ int paged_attn_launch(const void *q, const void *k_cache, const void *v_cache, c
                       const void *ctx_lens, float *out_f32, uint32_t *out_packed, _Float16 *out_q16, void *scratch,
                       int64_t n_seq,
                       int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
-                      int64_t max_ctx, int mode, float scale, hipStream_t s) {
+                      int64_t n_blocks, int64_t max_ctx, int mode, float scale, hipStream_t s) {
 #define FEATHER_PA(DD, MM)                                                                                           \
     return launch_paged<DD, MM>(q, k_cache, v_cache, block_tables, ctx_lens, out_f32, out_packed, out_q16, scratch,  \
-                                n_seq, n_q_heads, n_kv_heads, block_size, max_blocks, max_ctx, scale, s)
+                                n_seq, n_q_heads, n_kv_heads, block_size, max_blocks, n_blocks, max_ctx, scale, s)
     if (mode == FEATHER_E5M2) {
         if (d == 64) FEATHER_PA(64, FEATHER_E5M2);
         if (d == 128) FEATHER_PA(128, FEATHER_E5M2);
@@ -534,13 +538,16 @@ extern "C" int64_t feather_paged_attn_scratch_bytes(int64_t n_seq, int64_t n_q_h
 }
 
 extern "C" int feather_paged_attn_fp8(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,
-                                      const void *ctx_lens, void *out_f32, void *scratch, int64_t n_seq,
+                                      const void *ctx_lens, void *out_f32, void *out_packed, void *scratch, int64_t n_seq,
                                       int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size,
-                                      int64_t max_blocks, int64_t max_ctx, int mode, float scale, void *stream) {
+                                      int64_t max_blocks, int64_t n_blocks, int64_t max_ctx, int mode, float scale,
+                                      void *stream) {
     const char *me = "feather_paged_attn_fp8";
     FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE, "%s: mode %d not supported", me, mode);
     FEATHER_CHECK(n_seq >= 0 && n_q_heads > 0 && n_kv_heads > 0 && block_size > 0 && max_blocks >= 0 && max_ctx >= 0,
                   FEATHER_EINVAL, "%s: bad shape", me);
+    FEATHER_CHECK(n_blocks >= 1 && n_blocks < (1ll << 31), FEATHER_EINVAL, "%s: n_blocks=%lld: the cache must hold at least one block",
+                  me, (long long)n_blocks);
     FEATHER_CHECK(n_q_heads % n_kv_heads == 0, FEATHER_ESHAPE, "%s: n_q_heads=%lld not a multiple of n_kv_heads=%lld",
                   me, (long long)n_q_heads, (long long)n_kv_heads);
     FEATHER_CHECK(n_q_heads / n_kv_heads <= 16, FEATHER_ESHAPE, "%s: at most 16 query heads per KV head", me);
@@ -549,13 +556,14 @@ extern "C" int feather_paged_attn_fp8(const void *q, const void *k_cache, const 
     FEATHER_CHECK(max_ctx <= max_blocks * block_size, FEATHER_ESHAPE, "%s: max_ctx exceeds the block table", me);
     FEATHER_CHECK(scale > 0.f, FEATHER_EINVAL, "%s: scale must be positive (the running maximum is kept on raw scores)", me);
     if (n_seq == 0) return FEATHER_OK;
-    FEATHER_CHECK(q && k_cache && v_cache && block_tables && ctx_lens && out_f32 && scratch, FEATHER_EINVAL,
-                  "%s: null pointer", me);
-    FEATHER_CHECK(aligned(q, 8) && aligned(k_cache, 16) && aligned(v_cache, 16) && aligned(out_f32, 4) &&
-                      aligned(scratch, 16) && aligned(block_tables, 4) && aligned(ctx_lens, 4),
+    FEATHER_CHECK(q && k_cache && v_cache && block_tables && ctx_lens && scratch, FEATHER_EINVAL, "%s: null pointer", me);
+    FEATHER_CHECK(out_f32 || out_packed, FEATHER_EINVAL, "%s: no output (out_f32 and out_packed are both null)", me);
+    FEATHER_CHECK(aligned(q, 8) && aligned(k_cache, 16) && aligned(v_cache, 16) && aligned(out_f32, 16) &&
+                      aligned(out_packed, 4) && aligned(scratch, 16) && aligned(block_tables, 4) && aligned(ctx_lens, 4),
                   FEATHER_EINVAL, "%s: misaligned pointer", me);
-    return paged_attn_launch(q, k_cache, v_cache, block_tables, ctx_lens, (float *)out_f32, nullptr, nullptr, scratch, n_seq,
-                             n_q_heads, n_kv_heads, d, block_size, max_blocks, max_ctx, mode, scale, (hipStream_t)stream);
+    return paged_attn_launch(q, k_cache, v_cache, block_tables, ctx_lens, (float *)out_f32, (uint32_t *)out_packed, nullptr,
+                             scratch, n_seq, n_q_heads, n_kv_heads, d, block_size, max_blocks, n_blocks, max_ctx, mode, scale,
+                             (hipStream_t)stream);
 }
 
 // ---- the same attention for callers that cannot allocate -------------------------------------
@@ -592,9 +600,9 @@ static int pa_static_scratch(void **out, const char *me) {
 
 extern "C" int feather_paged_attn_fp8_static(const void *q, const void *k_cache, const void *v_cache,
                                              const void *block_tables, const void *ctx_lens, void *out_f32,
-                                             int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads, int64_t d,
-                                             int64_t block_size, int64_t max_blocks, int64_t max_ctx, int mode,
-                                             float scale, void *stream) {
+                                             void *out_packed, int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads,
+                                             int64_t d, int64_t block_size, int64_t max_blocks, int64_t n_blocks,
+                                             int64_t max_ctx, int mode, float scale, void *stream) {
     const char *me = "feather_paged_attn_fp8_static";
     const int64_t need = feather_paged_attn_scratch_bytes(n_seq, n_q_heads, d, max_ctx);
     FEATHER_CHECK(need <= (int64_t)FEATHER_PAGED_ATTN_STATIC_SCRATCH_BYTES, FEATHER_ESHAPE,
@@ -609,6 +617,6 @@ extern "C" int feather_paged_attn_fp8_static(const void *q, const void *k_cache,
     }
     // nothing in the buffer has to start at zero: the merge reads only the partials of splits that
     // hold tokens, and the split kernel of the same call writes exactly those
-    return feather_paged_attn_fp8(q, k_cache, v_cache, block_tables, ctx_lens, out_f32, scratch, n_seq, n_q_heads,
-                                  n_kv_heads, d, block_size, max_blocks, max_ctx, mode, scale, stream);
+    return feather_paged_attn_fp8(q, k_cache, v_cache, block_tables, ctx_lens, out_f32, out_packed, scratch, n_seq,
+                                  n_q_heads, n_kv_heads, d, block_size, max_blocks, n_blocks, max_ctx, mode, scale, stream);
 }

@@ -28,6 +28,7 @@ from __future__ import annotations
 
 import dataclasses
 import io
+import math
 import os
 import struct
 import zlib
@@ -121,7 +122,18 @@ def _read_record(f: BinaryIO, device) -> Union[None, Tuple[str, PackedTensor]]:
         raise NotImplementedError(f"mode code {mode} not supported")
     if rounding not in _ROUNDING_NAMES or ndim > 8 or name_len > 65535:
         raise ValueError("corrupt record header")
+    # the header is not covered by the checksum: check the word count against the shape and against
+    # what is left of the file before trusting it with a read
+    per = _PER_WORD[_MODE_NAMES[mode]]
+    if n_words != (n_elem + per - 1) // per or n_elem != math.prod(shape8[:ndim]):
+        raise ValueError("corrupt record header: element and word counts do not match the shape")
     name = _read_exact(f, name_len + _pad64(name_len), "name")[:name_len].decode("utf-8") if name_len else ""
+    if f.seekable():
+        here = f.tell()
+        left = f.seek(0, os.SEEK_END) - here
+        f.seek(here)
+        if 4 * n_words > left:
+            raise ValueError(f"truncated file: record {name!r} claims {4 * n_words} payload bytes, {left} remain")
     payload = _read_exact(f, 4 * n_words + _pad64(4 * n_words), "payload")[:4 * n_words]
     if zlib.crc32(payload) & 0xFFFFFFFF != crc:
         raise ValueError(f"checksum mismatch in record {name!r}")

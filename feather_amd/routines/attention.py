@@ -56,6 +56,8 @@ def flash_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: torch.
         raise ValueError("q, k and v must be on the same device")
     if scale is None:
         scale = 1.0 / math.sqrt(d)
+    if not scale > 0:
+        raise ValueError(f"scale must be positive, got {scale}")
     out = torch.empty((n_heads, seq_len, d), dtype=torch.float32, device=q.device)
     if causal:
         if tail != "mask":
@@ -116,6 +118,8 @@ def flash_attention_fp8_varlen_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v:
         raise ValueError(f"max_seqlen={max_seqlen} outside [0, total_rows={total}]")
     if scale is None:
         scale = 1.0 / math.sqrt(d)
+    if not scale > 0:
+        raise ValueError(f"scale must be positive, got {scale}")
     out = torch.zeros((n_heads, total, d), dtype=torch.float32, device=q.device)
     cu_seqlens = cu_seqlens.contiguous()
     N.call(q.device, "feather_flash_attn_fp8_varlen", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(cu_seqlens), cu_seqlens.numel() - 1, max_seqlen, total, n_heads, d, n_heads // n_kv, code, float(scale), 1 if causal else 0)

@@ -56,6 +56,8 @@ class PackedDecoder:
                  device=None):
         self.cfg, self.mode, self.code = cfg, mode, N.mode_code(mode)
         self.device = torch.device(device) if device is not None else N.require_gpu()
+        if self.device.type == "cuda" and self.device.index is None:
+            self.device = torch.device("cuda", torch.cuda.current_device())
         if cfg.hidden != cfg.n_q_heads * cfg.head_dim:
             raise ValueError("hidden must equal n_q_heads * head_dim")
         self.n_blocks, self.max_blocks = int(n_blocks), int(max_blocks)
@@ -85,7 +87,7 @@ class PackedDecoder:
             for name in ("w_qkv", "w_o", "w_gate_up", "w_down", "norm_attn", "norm_mlp", "k_cache", "v_cache"):
                 setattr(self._c_layers[i], name, lay[name].data_ptr())
         self._c = N.Decoder(cfg.n_layers, cfg.hidden, cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.inter, cfg.vocab,
-                            cfg.block_size, self.max_blocks, self.code, cfg.rms_eps, cfg.rope_theta,
+                            cfg.block_size, self.max_blocks, self.n_blocks, self.code, cfg.rms_eps, cfg.rope_theta,
                             ctypes.cast(self._c_layers, ctypes.POINTER(N.DecoderLayer)), self.embed.data_ptr(),
                             self.norm_final.data_ptr(), self.lm_head.data_ptr())
         self._scratch = {}
@@ -98,20 +100,35 @@ class PackedDecoder:
         return n
 
     def step(self, token_ids: torch.Tensor, block_tables: torch.Tensor, ctx_lens: torch.Tensor,
-             max_ctx: int | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+             max_ctx: int | None = None, out: torch.Tensor | None = None,
+             status: torch.Tensor | None = None) -> torch.Tensor:
         """Run one token for every sequence of the batch; returns float32 logits ``[batch, vocab]``.
         ``ctx_lens[b]`` is the number of tokens already cached for sequence ``b`` (the new token is
         written at that position; the caller adds 1 afterwards).  ``max_ctx`` bounds
-        ``ctx_lens + 1`` (default: the whole block table)."""
+        ``ctx_lens + 1`` (default: the whole block table).  ``status`` (optional int32 ``[batch]``)
+        receives 0 for every sequence whose token was appended, 1 where the block table is full or the
+        length negative, 2 where the table entry is not a block of the cache; those sequences are not
+        written and their logits are meaningless."""
         cfg = self.cfg
-        for t, name in ((token_ids, "token_ids"), (block_tables, "block_tables"), (ctx_lens, "ctx_lens")):
-            if t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous():
+        for t, name in ((token_ids, "token_ids"), (block_tables, "block_tables"), (ctx_lens, "ctx_lens"),
+                        (status, "status")):
+            if t is None:
+                continue
+            if not isinstance(t, torch.Tensor) or t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous():
                 raise ValueError(f"{name} must be a contiguous int32 tensor on the device")
+            if t.device != self.device:
+                raise ValueError(f"{name} is on {t.device}, the decoder on {self.device}")
         batch = token_ids.numel()
         if not 1 <= batch <= 64:
             raise ValueError(f"batch must be in [1, 64], got {batch}")
         if block_tables.shape != (batch, self.max_blocks) or ctx_lens.shape != (batch,):
             raise ValueError("block_tables must be [batch, max_blocks] and ctx_lens [batch]")
+        if status is not None and status.shape != (batch,):
+            raise ValueError("status must be [batch]")
+        if out is not None:
+            if (not isinstance(out, torch.Tensor) or out.dtype != torch.float32 or not out.is_cuda
+                    or out.device != self.device or not out.is_contiguous() or tuple(out.shape) != (batch, cfg.vocab)):
+                raise ValueError(f"out must be a contiguous float32 [batch={batch}, vocab={cfg.vocab}] tensor on {self.device}")
         max_ctx = self.max_blocks * cfg.block_size if max_ctx is None else int(max_ctx)
         # one scratch buffer per (shape, stream): steps on different streams may run concurrently
         key = (batch, max_ctx, N.stream_ptr(self.device))
@@ -126,7 +143,7 @@ class PackedDecoder:
         if out is None:
             out = torch.empty((batch, cfg.vocab), dtype=torch.float32, device=self.device)
         N.call(self.device, "feather_decode_step", ctypes.addressof(self._c), N.ptr(token_ids), N.ptr(block_tables),
-               N.ptr(ctx_lens), batch, max_ctx, sptr, N.ptr(out))
+               N.ptr(ctx_lens), batch, max_ctx, sptr, N.ptr(out), N.ptr(status) if status is not None else None)
         return out
 
 

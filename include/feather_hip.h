@@ -65,6 +65,13 @@ const char *feather_last_error(void);
  * src must be 2-byte aligned, dst 4-byte aligned. */
 int feather_pack_fp8(const void *src_f16, void *dst_u32, int64_t n, int mode, int rounding, void *stream);
 
+/* fp32[n] -> u32[ceil(n/4)]: each value rounded fp32 -> fp16 -> FP8 (round to nearest even twice,
+ * i.e. pack_fp8_tensor applied to x.half()), tail padded with +0.  No reference counterpart: the
+ * reference packs on the CPU from fp16 (feather/packers/fp8.py:260-281); this is the rounding chain
+ * every fp32 producer that feeds a packed GEMV uses (the norm, SwiGLU, rotary and attention
+ * epilogues below), as an operation of its own. */
+int feather_quant_pack_f32(const void *src_f32, void *dst_u32, int64_t n, int mode, void *stream);
+
 /* u32[n_words] -> fp32 or fp16 [4 * n_words] in element order.
  * Replaces unpack_fp8_from_fp32 / unpack_into_fp8_ndarray
  * (feather/packers/fp8.py:336-392, :395-432) with semantics = IEEE, the legacy
@@ -95,6 +102,15 @@ int feather_gemv_fp8(const void *m, const void *v, void *out_f32, int64_t M, int
 int feather_gemv_fp8_batched(const void *w, const void *x, void *out_f32, int64_t M, int64_t K, int64_t nvec, int mode,
                              void *stream);
 
+/* act[b, i] = silu(g) * u with g = sum_k dec(w[i, k]) dec(x[b, k]), u = sum_k dec(w[inter + i, k]) dec(x[b, k]),
+ * written as packed FP8 words act_packed [nvec, inter / 4] (fp32 -> fp16 -> FP8 as feather_quant_pack_f32)
+ * and, if act_f32 is not NULL, also as the fp32 values [nvec, inter] the codes were rounded from.
+ * w_gate_up is [2 * inter, K] packed: gate rows, then up rows.  silu(g) = g / (1 + 2^(-g log2 e)) with the
+ * hardware exp2 and reciprocal.  K % 256 == 0, inter % 4 == 0, 1 <= nvec <= 64, 16-byte aligned w and x.
+ * No reference counterpart (quantise + pack fused into the producing GEMV). */
+int feather_gemv_fp8_batched_swiglu(const void *w_gate_up, const void *x, void *act_packed, void *act_f32, int64_t inter,
+                                    int64_t K, int64_t nvec, int mode, void *stream);
+
 /* Bytes of scratch feather_dot_* need (one buffer per stream in flight; 64-byte
  * aligned; contents need no initialisation). */
 int64_t feather_dot_scratch_bytes(void);
@@ -119,7 +135,7 @@ int feather_dot_fp16(const void *x1, const void *x2, void *out_f32, void *scratc
  * independent heads, out[h] = softmax(Q K^T * scale) V, Q/K/V [L, d/4] words,
  * out [L, d] fp32; scores fp32, P rounded to fp16 before P.V, fp32 output.
  * d in {64, 128, 256, 512}.  kv_group > 1 maps query head h to K/V head
- * h / kv_group (K/V then hold n_heads / kv_group heads).
+ * h / kv_group (K/V then hold n_heads / kv_group heads).  scale must be positive.
  * Replaces flash_attention_fp8_e5m2_acc_fp32_gpu
  * (feather/routines/attention.py:110-179) at n_heads = 1, mode = E5M2,
  * scale = 1/sqrt(d), tail = REFERENCE. */
@@ -132,7 +148,9 @@ int feather_flash_attn_fp8(const void *q, const void *k, const void *v, void *ou
  *   q            [n_heads, total_rows, d/4] words; k, v [n_heads / kv_group, total_rows, d/4]
  *   cu_seqlens   [n_seq + 1] int32 on the device, non-decreasing row offsets: sequence s is
  *                rows cu[s] .. cu[s+1]-1 of every head and attends only to itself
- *   max_seqlen   upper bound of cu[s+1] - cu[s] (sizes the grid; rows past it are not computed)
+ *   max_seqlen   upper bound of cu[s+1] - cu[s]: it sizes the grid, so rows of a sequence beyond its first
+ *                max_seqlen rows are NOT computed and keep whatever `out` held (the caller must pass a
+ *                true bound; the kernel cannot report a longer sequence)
  *   out          [n_heads, total_rows, d] fp32; rows outside every sequence are left untouched
  *   causal       1: query i of a sequence sees keys 0..i of that sequence
  * A fixed-length batch is n_seq = 1, cu = {0, L}, n_heads = batch * heads. */
@@ -148,12 +166,13 @@ int feather_flash_attn_fp8_varlen(const void *q, const void *k, const void *v, v
  *   k_cache       [n_blocks, n_kv_heads, block_size, d/4] words (v_cache same)
  *   block_tables  [n_seq, max_blocks] int32; cu_seqlens [n_seq + 1] int32
  *   start_pos     [n_seq] int32 or NULL (all 0): cache position of each sequence's first row
- * Row cu[s] + i goes to position start_pos[s] + i of sequence s.  Positions at or beyond
- * max_blocks * block_size have no table entry and are dropped.  d % 16 == 0. */
+ * Row cu[s] + i goes to position start_pos[s] + i of sequence s.  Positions below 0 or at or beyond
+ * max_blocks * block_size have no table entry and are dropped, and so are rows whose table entry
+ * is not a block of the cache (outside [0, n_blocks): padding, -1).  d % 16 == 0. */
 int feather_paged_cache_write(const void *k_src, const void *v_src, int src_f16, void *k_cache, void *v_cache,
                               const void *block_tables, const void *cu_seqlens, const void *start_pos, int64_t n_seq,
                               int64_t total_rows, int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
-                              int mode, void *stream);
+                              int64_t n_blocks, int mode, void *stream);
 
 /* Bytes of scratch feather_paged_attn_fp8 needs for the given problem. */
 int64_t feather_paged_attn_scratch_bytes(int64_t n_seq, int64_t n_q_heads, int64_t d, int64_t max_ctx);
@@ -163,12 +182,17 @@ int64_t feather_paged_attn_scratch_bytes(int64_t n_seq, int64_t n_q_heads, int64
  *   q            [n_seq, n_q_heads, d/4] words
  *   k_cache      [n_blocks, n_kv_heads, block_size, d/4] words (v_cache same)
  *   block_tables [n_seq, max_blocks] int32, ctx_lens [n_seq] int32
- *   out          [n_seq, n_q_heads, d] fp32
- * Query head h uses KV head h / (n_q_heads / n_kv_heads). */
+ *   out_f32      [n_seq, n_q_heads, d] fp32, and / or
+ *   out_packed   [n_seq, n_q_heads * d / 4] words: the same result rounded fp32 -> fp16 -> FP8 of `mode`
+ *                (as feather_quant_pack_f32), the packed operand of a following GEMV; either may be NULL
+ * Query head h uses KV head h / (n_q_heads / n_kv_heads).  Table entries of positions below
+ * ctx_lens[s] must be blocks of the cache; an entry outside [0, n_blocks) is read as the last block
+ * (a wrong result for that sequence, never an access outside the cache).  Entries past the context
+ * are not used.  Negative context lengths count as 0 (a zero result). */
 int feather_paged_attn_fp8(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,
-                           const void *ctx_lens, void *out_f32, void *scratch, int64_t n_seq, int64_t n_q_heads,
-                           int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks, int64_t max_ctx,
-                           int mode, float scale, void *stream);
+                           const void *ctx_lens, void *out_f32, void *out_packed, void *scratch, int64_t n_seq,
+                           int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
+                           int64_t n_blocks, int64_t max_ctx, int mode, float scale, void *stream);
 
 /* feather_paged_attn_fp8 for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.
@@ -181,9 +205,10 @@ int feather_paged_attn_fp8(const void *q, const void *k_cache, const void *v_cac
  * the buffer needs clearing between calls.  Results are bit-identical to feather_paged_attn_fp8. */
 #define FEATHER_PAGED_ATTN_STATIC_SCRATCH_BYTES (4 << 20)
 int feather_paged_attn_fp8_static(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,
-                                  const void *ctx_lens, void *out_f32, int64_t n_seq, int64_t n_q_heads,
-                                  int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
-                                  int64_t max_ctx, int mode, float scale, void *stream);
+                                  const void *ctx_lens, void *out_f32, void *out_packed, int64_t n_seq,
+                                  int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size,
+                                  int64_t max_blocks, int64_t n_blocks, int64_t max_ctx, int mode, float scale,
+                                  void *stream);
 
 /* ---- decode step of a Llama-shaped model on packed weights (no reference counterpart) ----
  *
@@ -210,6 +235,7 @@ typedef struct feather_decoder_layer {
 typedef struct feather_decoder {
     int32_t n_layers, hidden, n_q_heads, n_kv_heads, head_dim, inter, vocab;
     int32_t block_size, max_blocks; /* KV paging: block_tables is [batch, max_blocks] */
+    int32_t n_blocks;               /* blocks in every layer's k_cache / v_cache */
     int32_t mode;                   /* FEATHER_E5M2 / FEATHER_E4M3 for weights, activations and cache */
     float rms_eps, rope_theta;
     const feather_decoder_layer_t *layers; /* host array of n_layers entries */
@@ -223,9 +249,39 @@ int64_t feather_decode_step_scratch_bytes(const feather_decoder_t *dec, int64_t 
 
 /* token_ids [batch] int32, block_tables [batch, max_blocks] int32, ctx_lens [batch] int32 (tokens
  * already in the cache; the caller adds 1 after the step), logits [batch, vocab] fp32.
- * batch <= 64; max_ctx bounds ctx_lens + 1. */
+ * batch <= 64; max_ctx bounds ctx_lens + 1.
+ * seq_status [batch] int32 or NULL: 0 = the new token's K/V were appended; 1 = ctx_lens[b] is negative
+ * or the block table is full (>= max_blocks * block_size); 2 = the table entry of the new position is
+ * not a block of the cache (outside [0, n_blocks)).  With 1 or 2 nothing is written to the cache for
+ * that sequence and its logits come from the tokens already cached: the caller must not use them. */
 int feather_decode_step(const feather_decoder_t *dec, const void *token_ids, const void *block_tables,
                         const void *ctx_lens, int64_t batch, int64_t max_ctx, void *scratch, void *logits_f32,
+                        void *seq_status, void *stream);
+
+/* The fused producers of the decode step as operations of their own (no reference counterpart: the
+ * reference has no device-side quantisation; they are the callers' side of the packed GEMV, where the
+ * fp32 -> FP8 rounding and the packing happen in the kernel that produces the values).
+ *
+ * feather_add_rmsnorm_pack: for each of `batch` rows, h += sum of the n_part slices of delta (slice s at
+ * delta + s * part_stride floats, [batch, hidden] each, added in slice order; delta may be NULL), then
+ * y = h * (1 / sqrt(mean(h^2) + eps)) * gain and xq = packed FP8 of y ([batch, hidden / 4] words).
+ * y_f32 (optional, [batch, hidden]) receives the fp32 values the codes were rounded from.  hidden % 4 == 0. */
+int feather_add_rmsnorm_pack(void *h_f32, const void *delta_f32, int64_t n_part, int64_t part_stride,
+                             const void *gain_f32, void *xq_u32, void *y_f32, int64_t batch, int64_t hidden, float eps,
+                             int mode, void *stream);
+
+/* feather_rope_append: qkv [batch, (n_q + 2 n_kv) * d] fp32 (q heads, k heads, v heads; given as n_part
+ * slices part_stride floats apart that are added in slice order) -> rotary embedding at position
+ * ctx_lens[b] on the q and k heads (rotate-half: element j pairs with j + d/2, angle pos * theta^(-2j/d)),
+ * q written as packed FP8 words q_packed [batch, n_q, d/4], k and v encoded and appended to the paged
+ * cache ([n_blocks, n_kv, block_size, d/4] words) at position ctx_lens[b] through block_tables
+ * [batch, max_blocks]; ctx_after[b] = ctx_lens[b] + 1.  seq_status (optional) as in feather_decode_step:
+ * a token without a valid slot is not written and ctx_after[b] keeps the old length.  rot_f32 (optional,
+ * [batch, n_q + 2 n_kv, d]) receives the fp32 values the codes were rounded from.  d % 8 == 0. */
+int feather_rope_append(const void *qkv_f32, int64_t n_part, int64_t part_stride, const void *ctx_lens,
+                        const void *block_tables, void *q_packed, void *k_cache, void *v_cache, void *ctx_after,
+                        void *seq_status, void *rot_f32, int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t d,
+                        int64_t block_size, int64_t max_blocks, int64_t n_blocks, float rope_theta, int mode,
                         void *stream);
 
 #ifdef __cplusplus

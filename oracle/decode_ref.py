@@ -124,14 +124,13 @@ def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables
                 v_caches[l][blk, kvh, slot] = store(v[kvh])
             qd = quant(q, mode)
             n = pos + 1
-            for hq in range(nq):
-                kvh = hq // (nq // nkv)
-                rows = [(int(block_tables[b][t // cfg.block_size]), t % cfg.block_size) for t in range(n)]
-                Kw = np.stack([k_caches[l][bb, kvh, ss] for bb, ss in rows])
-                Vw = np.stack([v_caches[l][bb, kvh, ss] for bb, ss in rows])
-                Kd = load(Kw, n, d)
-                Vd = load(Vw, n, d)
-                attn[b, hq * d:(hq + 1) * d] = online_attention(Kd @ qd[hq], Vd, float(scale))
+            t = np.arange(n)
+            blocks, slots = np.asarray(block_tables[b])[t // cfg.block_size], t % cfg.block_size
+            for kvh in range(nkv):
+                Kd = load(k_caches[l][blocks, kvh, slots], n, d)
+                Vd = load(v_caches[l][blocks, kvh, slots], n, d)
+                for hq in range(kvh * (nq // nkv), (kvh + 1) * (nq // nkv)):     # query head hq reads KV head hq // group
+                    attn[b, hq * d:(hq + 1) * d] = online_attention(Kd @ qd[hq], Vd, float(scale))
         o = (quant(attn, mode) @ Wq(g("wo")).T).astype(np.float32)
         h = h + o
         xq = quant(rmsnorm(h, g("norm_mlp"), cfg.rms_eps), mode)

@@ -131,7 +131,8 @@ def test_flash_attention_e5m2_subnormal_codes_count(dev, orc, d):
 
 def test_flash_attention_config_sized_property(dev):
     """B4 H16 L4096 d64 E5M2: too big for the scalar oracle; compare with torch SDPA (fp32
-    math) of the decoded operands on device and check determinism."""
+    math) of the operands decoded by the HIP unpack kernel (bit-exact to the oracle's decode on all
+    256 codes, test_gpu_pack.py) on device and check determinism."""
     import feather_amd as feather
     g = torch.Generator().manual_seed(3)
     B, H, L, d = 4, 16, 4096, 64
@@ -156,11 +157,16 @@ def test_flash_attention_config_sized_property(dev):
     ("E5M2", 1, 8, 4096, 256, False), ("E4M3", 1, 8, 1024, 256, False),
     # d = 256 with >= 256 workgroups of 256 queries: 32 queries per wave
     ("E4M3", 2, 16, 2048, 256, False), ("E5M2", 2, 16, 2048, 256, True), ("E4M3", 1, 8, 8192, 256, False),
+    # the wide-head benchmark configuration (B1 H8, E4M3) at its two remaining lengths
+    ("E4M3", 1, 8, 1024, 512, False), ("E4M3", 1, 8, 4096, 512, False),
+    ("E5M2", 4, 16, 4096, 64, False),
 ])
 def test_flash_attention_full_size_rows_vs_fp32_math(dev, mode, B, H, L, d, causal):
     """The remaining attention shapes of the benchmark configurations, too big for the scalar oracle:
     a sample of query rows of two heads against explicit fp32 softmax(q K^T / sqrt(d)) V of the
-    decoded operands (float64 accumulation on the device)."""
+    decoded operands (float64 accumulation on the device).  The operands are decoded by the HIP unpack
+    kernel, which test_gpu_pack.py holds bit-exact to the oracle's decode on all 256 codes of both modes
+    in the same run."""
     import feather_amd as feather
     g = torch.Generator(device=dev).manual_seed(L + d)
     qkv = [torch.randn(B, H, L, d, generator=g, device=dev).half() for _ in range(3)]

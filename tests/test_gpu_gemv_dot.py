@@ -104,7 +104,9 @@ def test_gemv_e4m3_uses_kernel_decode_not_ieee(dev, orc):
 
 def test_gemv_config_sized_properties(dev):
     """16384 x 16384 (too large for the scalar oracle): linearity in the vector and agreement
-    with a torch fp32 matvec of the decoded operands, both on device."""
+    with a torch float64 matvec of the operands decoded by the HIP unpack kernel, both on device.  That
+    check leans on the unpack kernel, which test_gpu_pack.py holds bit-exact to the oracle's decode on
+    all 256 codes of both modes in the same run."""
     import feather_amd as feather
     g = torch.Generator().manual_seed(2)
     M = K = 16384
@@ -159,7 +161,8 @@ def test_gemv_batched_vs_oracle(dev, orc, mode, M, K, nvec):
 @pytest.mark.parametrize("M,K", [(32000, 2048), (11264, 2048), (2048, 5632), (2560, 2048)])
 def test_gemv_batched_decode_shapes_vs_fp64_math(dev, M, K):
     """The weight shapes of the TinyLlama-shaped decode step at batch 32, E4M3: against a float64
-    matmul of the decoded operands on the device (the scalar oracle is too slow here)."""
+    matmul of the operands decoded by the HIP unpack kernel on the device (the scalar oracle is too slow
+    here; the unpack kernel is held bit-exact to the oracle's decode on all 256 codes by test_gpu_pack.py)."""
     import feather_amd as feather
     from feather_amd.routines.gemv import gemv_fp8_batched_acc_fp32_gpu
     g = torch.Generator(device=dev).manual_seed(M + K)
@@ -288,6 +291,56 @@ def test_dot_fp8_vs_oracle(dev, orc, mode, n):
     assert abs(got - orc.dot_fp8(x1, x2, mode, acc64=True)) <= 1e-5 * norm
     again = feather.dot(_dev_words(x1, dev), _dev_words(x2, dev), mode=mode).item()
     assert again == got                                        # deterministic reduction order
+
+
+@pytest.mark.parametrize("mode", ["E4M3", "E5M2"])
+def test_dot_config_size_2_pow_24_vs_oracle(dev, orc, mode):
+    """n = 2^24 with 1 % of the entries scaled by 1e-3 (E4M3 subnormal codes): the launch of 1024
+    workgroups plus the ordered finish over 1024 partials, against the C oracle's O(n) loop with a
+    float64 accumulator (reference semantics: dot.py:145-192 decode and products, summation order
+    free) and against the LUT decode + float64 BLAS reduction."""
+    import feather_amd as feather
+    n = 1 << 24
+    rng = np.random.default_rng(24)
+    a = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    a[rng.random(n) < 0.01] *= 1e-3
+    b[rng.random(n) < 0.01] *= 1e-3
+    x1, x2 = orc.pack_fp8(a.astype(np.float16), mode), orc.pack_fp8(b.astype(np.float16), mode)
+    d1, d2 = orc.decode_np(x1, mode), orc.decode_np(x2, mode)
+    norm = float(np.abs(d1 * d2).sum())
+    want = float(orc.dot_fp8(x1, x2, mode, acc64=True))
+    assert abs(want - float(d1 @ d2)) <= 1e-9 * norm              # the two oracles agree
+    t1, t2 = _dev_words(x1, dev), _dev_words(x2, dev)
+    got = feather.dot(t1, t2, mode=mode).item()
+    assert abs(got - want) <= 1e-6 * norm                         # fp32 partial sums of 16384 terms each
+    assert abs(got - want) <= TOL * max(abs(want), 1e-3 * norm)
+    assert feather.dot(t1, t2, mode=mode).item() == got           # deterministic
+
+
+def test_gemv_config_size_8192_vs_oracle(dev, orc):
+    """BASELINE config 1 at its own size: E5M2, 8192 x 8192 N(0,1) from seed 1.  The scalar oracle
+    checks a sample of rows (every 64th plus the last); all rows are checked against a float64 matvec
+    of the operands decoded by the HIP unpack kernel, which the pack tests of the same run hold
+    bit-exact to the oracle's decode on all 256 codes."""
+    import feather_amd as feather
+    g = torch.Generator().manual_seed(1)
+    M = K = 8192
+    m = torch.randn(M, K, generator=g).half()
+    v = torch.randn(K, generator=g).half()
+    mp = feather.pack_fp8_tensor(m.to(dev), mode="E5M2")
+    vp = feather.pack_fp8_tensor(v.to(dev), mode="E5M2")
+    out = feather.gemv(mp, vp, original_shape=(M, K), mode="E5M2")
+    rows = np.r_[0:M:64, M - 1]
+    mw = mp.view(torch.int32).cpu().numpy().view(np.uint32).reshape(M, K // 4)
+    assert np.array_equal(mw[rows], orc.pack_fp8(m.numpy()[rows], "E5M2").reshape(len(rows), K // 4))   # packing bit-exact
+    vw = vp.view(torch.int32).cpu().numpy().view(np.uint32)
+    want = orc.gemv(np.ascontiguousarray(mw[rows]).reshape(-1), vw, len(rows), K, "E5M2", acc64=True)
+    full = torch.mv(feather.unpack_fp8_tensor(mp, mode="E5M2", semantics="kernel").view(M, K).double(),
+                    feather.unpack_fp8_tensor(vp, mode="E5M2", semantics="kernel").double())
+    scale = full.abs().max().item()
+    assert np.abs(out.cpu().numpy()[rows] - want).max() / scale <= 1e-5
+    assert ((out.double() - full).abs().max() / scale).item() <= 1e-5
 
 
 @pytest.mark.parametrize("n", [2, 1001, 1 << 20])

@@ -59,8 +59,35 @@ def test_c_abi_argument_checks_without_gpu():
     assert L.feather_flash_attn_fp8(None, None, None, None, 1, 64, 64, 1, N.E5M2, 0.1, 5, None) == N.EINVAL
     assert L.feather_unpack_fp8(None, None, 4, N.E5M2, 9, 0, 0, None) == N.EINVAL
     assert L.feather_dot_fp8(None, None, None, None, 4, 2, None) == N.EMODE
-    assert L.feather_paged_attn_fp8(None, None, None, None, None, None, None, 1, 6, 4, 64, 16, 4, 64, N.E5M2, 0.1,
-                                    None) == N.ESHAPE
+    assert L.feather_paged_attn_fp8(None, None, None, None, None, None, None, None, 1, 6, 4, 64, 16, 4, 8, 64, N.E5M2,
+                                    0.1, None) == N.ESHAPE
+    assert L.feather_paged_attn_fp8(None, None, None, None, None, None, None, None, 1, 8, 4, 64, 16, 4, 0, 64, N.E5M2,
+                                    0.1, None) == N.EINVAL                           # a cache without blocks
+    assert L.feather_paged_attn_fp8_static(None, None, None, None, None, None, None, 64, 64, 4, 128, 16, 512, 9, 8192,
+                                           N.E4M3, 0.1, None) == N.ESHAPE            # partials beyond the built-in buffer
+    assert b"built-in buffer" in L.feather_last_error()
+    # a zero or negative softmax scale is rejected everywhere (the running maximum is kept on raw scores)
+    assert L.feather_flash_attn_fp8(None, None, None, None, 1, 64, 64, 1, N.E5M2, 0.0, 0, None) == N.EINVAL
+    assert L.feather_flash_attn_fp8(None, None, None, None, 1, 64, 64, 1, N.E5M2, -0.125, 0, None) == N.EINVAL
+    assert b"scale" in L.feather_last_error()
+    assert L.feather_flash_attn_fp8_varlen(None, None, None, None, None, 1, 64, 64, 1, 64, 1, N.E5M2, -1.0, 0,
+                                           None) == N.EINVAL
+    assert L.feather_paged_attn_fp8(None, None, None, None, None, None, None, None, 1, 8, 4, 64, 16, 4, 8, 64, N.E5M2,
+                                    0.0, None) == N.EINVAL
+    # the fused producers
+    assert L.feather_quant_pack_f32(None, None, 8, 5, None) == N.EMODE
+    assert L.feather_quant_pack_f32(None, None, 8, N.E4M3, None) == N.EINVAL
+    assert L.feather_quant_pack_f32(None, None, 0, N.E4M3, None) == N.OK
+    assert L.feather_add_rmsnorm_pack(None, None, 0, 0, None, None, None, 2, 30, 1e-5, N.E4M3, None) == N.ESHAPE
+    assert L.feather_add_rmsnorm_pack(None, None, 0, 0, None, None, None, 2, 32, 1e-5, N.E4M3, None) == N.EINVAL
+    assert L.feather_gemv_fp8_batched_swiglu(None, None, None, None, 64, 100, 4, N.E4M3, None) == N.ESHAPE
+    assert L.feather_gemv_fp8_batched_swiglu(None, None, None, None, 64, 256, 65, N.E4M3, None) == N.ESHAPE
+    assert L.feather_rope_append(None, 1, 0, None, None, None, None, None, None, None, None, 2, 4, 2, 60, 16, 4, 8,
+                                 10000.0, N.E4M3, None) == N.ESHAPE
+    assert L.feather_rope_append(None, 1, 0, None, None, None, None, None, None, None, None, 2, 4, 2, 64, 16, 4, 0,
+                                 10000.0, N.E4M3, None) == N.EINVAL                  # n_blocks = 0
+    assert L.feather_paged_cache_write(None, None, 0, None, None, None, None, None, 1, 4, 2, 64, 16, 4, -1, N.E5M2,
+                                       None) == N.EINVAL
 
 
 def test_error_mapping():
@@ -95,6 +122,80 @@ def test_python_validation_before_any_device_work():
         feather.gemv(w, w, original_shape=(4, 8), mode="E2M5")
     with pytest.raises(ValueError):
         feather.gemv(w, w)
+
+
+def test_wrappers_reject_host_tensors_before_any_launch():
+    """A CPU tensor handed to a wrapper would reach the kernel as a host pointer (a GPU memory fault);
+    every wrapper must raise ValueError before the C ABI is called.  Runs without a GPU: nothing is launched."""
+    from feather_amd.routines import attention, producers
+    from feather_amd.routines.paged_attention import paged_attention_fp8_acc_fp32_gpu, paged_cache_write
+    w = lambda *s: torch.zeros(s, dtype=torch.int32)
+    i32 = lambda *s: torch.zeros(s, dtype=torch.int32)
+    kc = w(4, 2, 16, 16)
+    h16 = torch.zeros((2, 8, 64), dtype=torch.float16)
+    with pytest.raises(ValueError):                              # fp16 K/V on the host (the packed branch had this check already)
+        paged_cache_write(h16, h16, kc, kc, i32(1, 2), i32(2), mode="E5M2")
+    with pytest.raises(ValueError):
+        paged_cache_write(w(2, 8, 16), w(2, 8, 16), kc, kc, i32(1, 2), i32(2), mode="E5M2")
+    with pytest.raises(ValueError):
+        paged_attention_fp8_acc_fp32_gpu(w(1, 4, 16), kc, kc, i32(1, 2), i32(1), mode="E4M3")
+    with pytest.raises(ValueError):
+        producers.quant_pack_f32(torch.zeros(8))
+    with pytest.raises(ValueError):
+        producers.add_rmsnorm_pack(torch.zeros(2, 64), torch.ones(64))
+    with pytest.raises(ValueError):
+        producers.rope_append(torch.zeros(1, 8 * 64), i32(1), i32(1, 2), kc, kc, n_q_heads=4)
+    with pytest.raises(ValueError):
+        producers.gemv_fp8_batched_swiglu(w(2 * 8 * 256 // 4), w(256 // 4), 8, 256, 1)
+    with pytest.raises(ValueError):                              # non-positive softmax scale
+        attention.flash_attention_fp8_acc_fp32_gpu(w(64 * 16), w(64 * 16), w(64 * 16), 64, 16, scale=0.0)
+
+
+def test_decoder_step_validates_out_and_status_without_launching():
+    """PackedDecoder.step checks a caller-supplied `out` / `status` (device, dtype, shape, contiguity)
+    before the C call.  Exercised on an instance built without a device: validation comes first."""
+    from feather_amd.routines.decode import DecoderConfig, PackedDecoder
+    cfg = DecoderConfig(n_layers=1, hidden=256, n_q_heads=4, n_kv_heads=2, head_dim=64, inter=512, vocab=100)
+    dec = PackedDecoder.__new__(PackedDecoder)
+    dec.cfg, dec.device, dec.max_blocks, dec.n_blocks = cfg, torch.device("cuda", 0), 4, 8
+    tok = torch.zeros(2, dtype=torch.int32)
+    with pytest.raises(ValueError, match="token_ids"):           # host tensors never reach the library
+        dec.step(tok, torch.zeros((2, 4), dtype=torch.int32), tok)
+
+
+def test_cache_index_arithmetic_stays_inside_the_cache():
+    """CPU model of the device-side index arithmetic of the cache writers and readers
+    (csrc/kv_cache.hip, rope_append_kernel, paged_attn_split_kernel): whatever the table entries and
+    positions are -- negative, past the table, padding values -- every word offset that is written or
+    read lies inside [0, n_blocks * n_kv * block_size * dw)."""
+    rng = np.random.default_rng(3)
+    n_blocks, n_kv, bs, dw, max_blocks = 5, 2, 4, 16, 3
+    size = n_blocks * n_kv * bs * dw
+    cap = max_blocks * bs
+
+    def append_offset(pos_raw, blk):                             # rope_append_kernel / paged_cache_write_kernel
+        pos_ok = 0 <= pos_raw < cap
+        blk_ok = 0 <= blk < n_blocks
+        if not (pos_ok and blk_ok):
+            return None, (min(max(pos_raw, 0), cap), 1 if not pos_ok else 2)
+        return [((blk * n_kv + h) * bs + pos_raw % bs) * dw for h in range(n_kv)], (pos_raw + 1, 0)
+
+    def read_offset(blk, tok, kvh):                              # paged_attn_split_kernel: unsigned min with n_blocks - 1
+        b = min(blk & 0xFFFFFFFF, n_blocks - 1)
+        return ((b * n_kv + kvh) * bs + tok % bs) * dw
+
+    for pos_raw in (-7, -1, 0, 1, cap - 1, cap, cap + 5, 2**31 - 1):
+        for blk in (-2**31, -1, 0, n_blocks - 1, n_blocks, 10**6, 2**31 - 1):
+            offs, (ctx_after, status) = append_offset(pos_raw, blk)
+            if offs is None:
+                assert status in (1, 2) and 0 <= ctx_after <= cap
+            else:
+                assert status == 0 and ctx_after == pos_raw + 1 <= cap
+                assert all(0 <= o and o + dw <= size for o in offs)
+            for tok in range(cap):
+                for kvh in range(n_kv):
+                    o = read_offset(blk, tok, kvh)
+                    assert 0 <= o and o + dw <= size
 
 
 def test_no_cpu_fallback_when_no_device():

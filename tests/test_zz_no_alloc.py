@@ -37,14 +37,15 @@ def _run(P, static, dev):
     code = N.mode_code(P["mode"])
     scale = float(P["d"]) ** -0.5
     stream = N.stream_ptr(dev)
-    shape = (P["n_seq"], P["Hq"], P["Hkv"], P["d"], P["bs"], P["max_blocks"], P["max_ctx"], code, scale, stream)
+    n_blocks = P["kc"].numel() * 4 // (P["Hkv"] * P["bs"] * P["d"])
+    shape = (P["n_seq"], P["Hq"], P["Hkv"], P["d"], P["bs"], P["max_blocks"], n_blocks, P["max_ctx"], code, scale, stream)
     ptrs = [P[k].data_ptr() for k in ("q", "kc", "vc", "bt", "ctx")]
     if static:
-        rc = L.feather_paged_attn_fp8_static(*ptrs, out.data_ptr(), *shape)
+        rc = L.feather_paged_attn_fp8_static(*ptrs, out.data_ptr(), None, *shape)
     else:
         nbytes = int(L.feather_paged_attn_scratch_bytes(P["n_seq"], P["Hq"], P["d"], P["max_ctx"]))
         scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
-        rc = L.feather_paged_attn_fp8(*ptrs, out.data_ptr(), scratch.data_ptr(), *shape)
+        rc = L.feather_paged_attn_fp8(*ptrs, out.data_ptr(), None, scratch.data_ptr(), *shape)
     N.check(rc)
     torch.cuda.synchronize()
     return out.cpu().numpy()
@@ -69,7 +70,7 @@ def test_static_scratch_rejects_oversized_problem(dev):
     from feather_amd import _native as N
     L = N.lib()
     # 64 sequences x 64 heads x 16 splits x 130 floats = 34 MB of partials: more than the built-in 4 MiB
-    rc = L.feather_paged_attn_fp8_static(None, None, None, None, None, None, 64, 64, 4, 128, 16, 512, 8192, N.E4M3,
-                                         0.1, None)
+    rc = L.feather_paged_attn_fp8_static(None, None, None, None, None, None, None, 64, 64, 4, 128, 16, 512, 9, 8192,
+                                         N.E4M3, 0.1, None)
     assert rc == N.ESHAPE
     assert b"built-in buffer" in L.feather_last_error()

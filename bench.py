@@ -52,6 +52,50 @@ def gpu_time_us(fn, steps, warmup, sync, warm_ms=0.0):
     return start.elapsed_time(stop) * 1000.0 / steps
 
 
+def _source_hash(rel_paths) -> str:
+    """sha256 (first 16 hex digits) over the kernel sources a counter figure belongs to."""
+    import hashlib
+    h = hashlib.sha256()
+    for rel in rel_paths:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def load_traffic() -> dict:
+    """HBM bytes per launch from the committed rocprofv3 counter summary: lines
+    `hbm_bytes_per_launch <key> <bytes> <sha> <source>[,<source>...]`.  A figure whose kernel sources
+    have changed since the counters were taken is reported as stale (traffic = null) instead of being
+    carried along silently."""
+    out = {}
+    path = os.path.join(ROOT, "profiles", "bench_hbm_traffic.md")
+    if not os.path.exists(path):
+        return out
+    for ln in open(path):
+        f = ln.split()
+        if len(f) == 5 and f[0] == "hbm_bytes_per_launch":
+            try:
+                fresh = _source_hash(f[4].split(",")) == f[3]
+            except OSError:
+                fresh = False
+            out[f[1]] = (int(f[2]), fresh)
+    return out
+
+
+def roofline_record(traffic_table, key, kernel, algorithmic_bytes, us, launches_per_call=1):
+    """`roofline`-style record of an HBM-bound workload: achieved = algorithmic bytes / measured time."""
+    achieved = algorithmic_bytes / (us * 1e-6) / 1e9
+    t = traffic_table.get(key)
+    rec = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+           "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": t[0] if t and t[1] else None, "kernel": kernel,
+           "algorithmic_bytes": int(algorithmic_bytes), "us": round(us, 3)}
+    if t and not t[1]:
+        rec["traffic_note"] = "stale: the kernel source changed since the counters in profiles/bench_hbm_traffic.md were taken"
+    if launches_per_call != 1:
+        rec["launches_per_call"] = launches_per_call
+    return rec
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -103,6 +147,8 @@ def main() -> int:
     # (three back-to-back series of 200 launches measured 45.7, 43.9 and 43.0 us), so the same launches
     # run for ~50 ms before the W warm-up steps; the timed region stays exactly K steps.
     PREWARM = 1200
+    sync()
+    cold_us = gpu_time_us(gemv_step("E4M3"), args.steps, 0, sync)   # the first series of the process, no warm-up at all
     for i in range(PREWARM):
         gemv_step("E4M3")(i)
     # the whole timed region, bracketed by synchronize on both sides
@@ -120,7 +166,6 @@ def main() -> int:
     wall_ms = (time.perf_counter() - t0) * 1000.0
     kern_us = ev0.elapsed_time(ev1) * 1000.0 / args.steps
     ms_per_step = wall_ms / args.steps
-    achieved = gemv_bytes / (kern_us * 1e-6) / 1e9
 
     if args.calibrate_copy:
         src = torch.empty(M * K // 4, dtype=torch.int32, device=dev).fill_(1)
@@ -130,20 +175,44 @@ def main() -> int:
         sync()
         del src, dst
 
-    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summary file)
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "gemv_fp8_16384_hbm_traffic.md")
-    if os.path.exists(tpath):
-        for ln in open(tpath):
-            if ln.startswith("hbm_bytes_per_launch_e4m3:"):
-                traffic = int(ln.split(":")[1].strip())
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/bench_hbm_traffic.md)
+    ttab = load_traffic()
+    headline = roofline_record(ttab, "gemv_e4m3_16384", "gemv_fp8_kernel<E4M3>", gemv_bytes, kern_us)
 
-    extra = {}
+    extra = {"gemv_e4m3_16384_cold_first_series_us": round(cold_us, 2)}   # same kernel before the clocks are up
+    rl = {}                                                               # roofline records of the other HBM-bound workloads
     if not args.no_extra:
         # cache-resident figure (one matrix re-used): reported separately, never the headline
         one = mats["E4M3"][0]
         extra["gemv_e4m3_16384_same_buffer_us"] = round(
             gpu_time_us(lambda i: feather.gemv(one, vecs["E4M3"], original_shape=(M, K), mode="E4M3"), 100, 10, sync), 2)
+        # the reference harness's GEMV grid (benchmark/bench_gemv.py:14-15 and README.md:33-35: 4096^2, 8192^2,
+        # 16384 x 8192, 16384^2) in E4M3 first, on views into the four rotating 256 MiB buffers (>= 4 distinct operands
+        # of every shape, 1 GiB cycled), then the same in E5M2
+        from feather_amd.routines.gemv import gemv_fp8_batched_acc_fp32_gpu
+
+        def gemv_grid(mode):
+            bufs = mats[mode]
+            for (Ms, Ks) in ((4096, 4096), (8192, 8192), (16384, 8192)):
+                words = Ms * Ks // 4
+                per = (M * K // 4) // words
+                views = [b[i * words:(i + 1) * words] for b in bufs for i in range(per)]
+                vp = feather.pack_fp8_tensor(v16[:Ks], mode=mode)
+                us = gpu_time_us(lambda i: feather.gemv(views[i % len(views)], vp, original_shape=(Ms, Ks), mode=mode),
+                                 args.steps, args.warmup, sync, 10.0)
+                key = f"gemv_{mode.lower()}_{Ms}x{Ks}" if Ms != Ks else f"gemv_{mode.lower()}_{Ms}"
+                extra[key + "_us"] = round(us, 2)
+                extra[key + "_GBps"] = round((Ms * Ks + Ks + 4 * Ms) / us / 1e3, 1)
+                rl[key] = roofline_record(ttab, key, f"gemv_fp8_kernel<{mode}>", Ms * Ks + Ks + 4 * Ms, us)
+            # batched GEMV: the rotating matrices against 32 vectors (weights streamed once per batch)
+            xb = feather.pack_fp8_tensor(randn(32, K).half(), mode=mode)
+            us = gpu_time_us(lambda i: gemv_fp8_batched_acc_fp32_gpu(bufs[i % NBUF], xb, (M, K), 32, mode), 50, 10, sync)
+            key = f"gemv_batched_{mode.lower()}_16384_x32"
+            extra[key + "_us"] = round(us, 2)
+            extra[key + "_GBps"] = round((M * K + 32 * K + 4 * 32 * M) / us / 1e3, 1)
+            rl[key] = roofline_record(ttab, key, f"gemv_batched_kernel<{mode}>", M * K + 32 * K + 4 * 32 * M, us)
+
+        gemv_grid("E4M3")
         del mats["E4M3"]
         torch.cuda.empty_cache()
         mats["E5M2"] = [make_matrix("E5M2") for _ in range(NBUF)]
@@ -151,23 +220,8 @@ def main() -> int:
         extra["gemv_e5m2_16384_us"] = round(us, 2)
         extra["gemv_e5m2_16384_GBps"] = round(gemv_bytes / us / 1e3, 1)
         extra["gemv_e5m2_16384_hbm_frac"] = round(gemv_bytes / us / 1e3 / HBM_PEAK_GBS, 4)
-        # batched GEMV: the same rotating E5M2 matrices against 32 vectors (weights streamed once per batch)
-        from feather_amd.routines.gemv import gemv_fp8_batched_acc_fp32_gpu
-        xb = feather.pack_fp8_tensor(randn(32, K).half(), mode="E5M2")
-        us = gpu_time_us(lambda i: gemv_fp8_batched_acc_fp32_gpu(mats["E5M2"][i % NBUF], xb, (M, K), 32, "E5M2"),
-                         50, 10, sync)
-        extra["gemv_batched_e5m2_16384_x32_us"] = round(us, 2)
-        extra["gemv_batched_e5m2_16384_x32_GBps"] = round((M * K + 32 * K + 4 * 32 * M) / us / 1e3, 1)
-        del xb
-        # config 0: 8192 x 8192 E5M2 (views into the 16384^2 buffers: 4 distinct 64 MiB matrices each)
-        M0 = K0 = 8192
-        sub = [b[i * (M0 * K0 // 4):(i + 1) * (M0 * K0 // 4)] for b in mats["E5M2"] for i in range(4)]
-        v0 = feather.pack_fp8_tensor(v16[:K0], mode="E5M2")
-        us = gpu_time_us(lambda i: feather.gemv(sub[i % 16], v0, original_shape=(M0, K0), mode="E5M2"),
-                         args.steps, args.warmup, sync)
-        b0 = M0 * K0 + K0 + 4 * M0
-        extra["gemv_e5m2_8192_us"] = round(us, 2)
-        extra["gemv_e5m2_8192_GBps"] = round(b0 / us / 1e3, 1)
+        rl["gemv_e5m2_16384"] = roofline_record(ttab, "gemv_e5m2_16384", "gemv_fp8_kernel<E5M2>", gemv_bytes, us)
+        gemv_grid("E5M2")
         # dot, n = 2^24 (E4M3): rotate through the big buffers
         n = 1 << 24
         xs = [b[i * (n // 4):(i + 1) * (n // 4)] for b in mats["E5M2"] for i in range(16)]
@@ -176,6 +230,8 @@ def main() -> int:
                              args.warmup, sync)
             extra[f"dot_{mode.lower()}_2p24_us"] = round(us, 2)
             extra[f"dot_{mode.lower()}_2p24_GBps"] = round((2 * n + 4) / us / 1e3, 1)
+            rl[f"dot_{mode.lower()}_2p24"] = roofline_record(ttab, f"dot_{mode.lower()}_2p24", f"dot_kernel<{mode}> + dot_finish_kernel",
+                                                              2 * n + 4, us, launches_per_call=2)
         # dot, n = 16384 (one workgroup, one launch: latency bound)
         xs_s = [x[:4096] for x in xs]
         for mode in ("E4M3", "E5M2"):
@@ -187,18 +243,21 @@ def main() -> int:
         for mode in ("E5M2", "E4M3"):
             us = gpu_time_us(lambda i: feather.pack_fp8_tensor(src, mode=mode), 20, 3, sync)
             extra[f"pack_{mode.lower()}_134M_GBps"] = round(3 * src.numel() / us / 1e3, 1)
+            rl[f"pack_{mode.lower()}_134M"] = roofline_record(ttab, f"pack_{mode.lower()}_134M", f"pack_fp8_kernel<{mode}>", 3 * src.numel(), us)
         # unpack (1 B in, 4 B fp32 out per element), ReLU on packed E5M2, fp16 container (2 B in + 2 B out)
         from feather_amd.routines.activations import relu1d_fp8_ret_fp32_feather_gpu
         words = mats["E5M2"][0][: src.numel() // 4]
         for mode, sem in (("E4M3", "ieee"), ("E4M3", "kernel"), ("E5M2", "ieee")):
             us = gpu_time_us(lambda i: feather.unpack_fp8_tensor(words, mode=mode, semantics=sem), 20, 3, sync)
             extra[f"unpack_{mode.lower()}_{sem}_f32_134M_GBps"] = round(5 * src.numel() / us / 1e3, 1)
+            rl[f"unpack_{mode.lower()}_{sem}_134M"] = roofline_record(ttab, f"unpack_{mode.lower()}_{sem}_134M",
+                                                                       f"unpack_fp8_kernel<{mode}, {sem}>", 5 * src.numel(), us)
         us = gpu_time_us(lambda i: relu1d_fp8_ret_fp32_feather_gpu(words, src.numel()), 20, 3, sync)
         extra["relu_e5m2_f32_134M_GBps"] = round(5 * src.numel() / us / 1e3, 1)
         us = gpu_time_us(lambda i: feather.pack_fp16_tensor(src), 20, 3, sync)
         extra["pack_fp16_134M_GBps"] = round(4 * src.numel() / us / 1e3, 1)
         del src, words
-        del mats["E5M2"], sub, xs
+        del mats["E5M2"], xs
         torch.cuda.empty_cache()
         # flash attention, B4 H16 d64, E5M2, vs fp16 SDPA on the same GPU (both sides get WARM_MS of
         # back-to-back warm-up calls: the first tens of milliseconds of a series run below the sustained clock)
@@ -222,6 +281,13 @@ def main() -> int:
                 us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16, is_causal=True),
                                       10, 10, sync, WARM_MS)
                 extra[f"sdpa_causal_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
+            if L == 8192:   # the same shape with E4M3 codes (fp16 score product: the E4M3 kernel decode is not the matrix core's format)
+                pk4 = [feather.pack_fp8_tensor(t, mode="E4M3").view(B, H, L, d // 4) for t in qkv16]
+                us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk4[0], pk4[1], pk4[2], L, d // 4, mode="E4M3"),
+                                 10, 10, sync, WARM_MS)
+                extra[f"flash_attn_e4m3_b4h16_d64_L{L}_us"] = round(us, 1)
+                extra[f"flash_attn_e4m3_b4h16_d64_L{L}_TFLOPs"] = round(flops / us / 1e6, 1)
+                del pk4
             del qkv16, pk
         # wide heads: B1 H8, d = 256 / 512, E4M3, vs fp16 SDPA
         for d, L in ((256, 1024), (256, 4096), (256, 8192), (512, 1024), (512, 4096), (512, 8192)):
@@ -251,6 +317,9 @@ def main() -> int:
                                                                         max_context_len=c), 50, 5, sync)
             extra[f"paged_attn_e4m3_s32_h32kv4_d64_ctx{c}_us"] = round(us, 2)
             extra[f"paged_attn_e4m3_s32_h32kv4_d64_ctx{c}_GBps"] = round(2 * n_seq * Hkv * d * c / us / 1e3, 1)
+            rl[f"paged_attn_e4m3_ctx{c}"] = roofline_record(
+                ttab, f"paged_attn_e4m3_ctx{c}", "paged_attn_split_kernel<64, E4M3>" + (" + paged_attn_merge_kernel" if c > 512 else ""),
+                2 * n_seq * Hkv * d * c + n_seq * Hq * d * 5, us, launches_per_call=2 if c > 512 else 1)
         # prefill -> paged cache: 32 sequences x 2048 rows x 4 KV heads of packed K and V (1 B in + 1 B out per code)
         from feather_amd.routines.paged_attention import paged_cache_write
         rows = n_seq * 2048
@@ -284,6 +353,8 @@ def main() -> int:
             extra[key + "_ms_per_step"] = round(us / 1e3, 3)
             extra[key + "_tokens_per_s"] = round(batch / us * 1e6, 0)
             extra[key + "_GBps"] = round(step_bytes / us / 1e3, 1)
+            rl[key] = roofline_record(ttab, key, "feather_decode_step (all kernels of one step)", step_bytes, us,
+                                      launches_per_call=10 * cfg.n_layers + 3)
             del dec, logits, btd
             torch.cuda.empty_cache()
 
@@ -292,13 +363,15 @@ def main() -> int:
         from oracle import cpu_baseline
         r = cpu_baseline.gemv_baseline(M, K, "E4M3", sample_rows=2048, repeats=3)
         cpu = {"value": round(r["total_s"] * 1e6, 1), "unit": "us", "cores": r["cores"], "kind": "port",
-               "sample": r["sample"] + "; decode (LUT gather) + fp32 torch.mv, pack excluded",
+               "sample": r["sample"] + "; pack (torch-CPU float8 cast + byte assembly) + decode (LUT gather) + fp32 torch.mv, summed",
                "pack_us": round(r["pack_s"] * 1e6, 1), "decode_us": round(r["decode_s"] * 1e6, 1),
                "compute_us": round(r["compute_s"] * 1e6, 1), "cpu_count": r["cpu_count"]}
-        # second half of the metric: decode + fp32 SDPA per head (B4 H16 d=64 L=8192, E5M2), two heads timed
+        # second half of the metric: pack + decode + fp32 SDPA per head (B4 H16 d=64 L=8192, E5M2), two heads timed
         ra = cpu_baseline.attention_baseline(64, 8192, 64, "E5M2", sample_heads=2, repeats=3)
-        cpu["flash_attn_e5m2_b4h16_d64_L8192_us"] = round(ra["total_s"] * 1e6, 1)
-        cpu["flash_attn_sample"] = ra["sample"] + "; decode (LUT gather) + fp32 SDPA per head, median of 3"
+        cpu["flash_attn_e5m2_b4h16_d64_L8192"] = {
+            "value": round(ra["total_s"] * 1e6, 1), "unit": "us", "cores": ra["cores"], "kind": "port",
+            "sample": ra["sample"] + "; pack + decode (LUT gather) + fp32 SDPA per head, summed, median of 3",
+            "pack_us": round(ra["pack_s"] * 1e6, 1), "decode_and_sdpa_us": round(ra["compute_s"] * 1e6, 1)}
 
     line = {
         "metric": "packed-FP8 GEMV us (16384^2, E4M3, FP32 accumulate)",
@@ -309,12 +382,9 @@ def main() -> int:
                                "sources with 1% of entries x1e-3, packed 4 codes per 32-bit word; 4 distinct "
                                "matrices (1 GiB) rotated",
                    "M": M, "K": K, "mode": "E4M3", "buffers": NBUF, "clock_prewarm_launches": PREWARM},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "gemv_fp8_kernel<E4M3>", "algorithmic_bytes": gemv_bytes,
-                     "avg_launch_us": round(kern_us, 3)},
+        "roofline": dict(headline, avg_launch_us=round(kern_us, 3)),
         "cpu_baseline": cpu,
-        "extra": extra,
+        "extra": dict(extra, roofline=rl),
     }
     print(json.dumps(line))
     return 0

@@ -437,21 +437,42 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const float *__re
     const int gid = blockIdx.x * 256 + threadIdx.x;
     const int item = gid / DW, w4 = gid % DW;      // item = seq * n_q_heads + qh
     if (item >= n_items) return;
-    const int ctx = min(ctx_lens[item / n_q_heads], max_ctx);
-    const int used = min(n_splits, (ctx + kSplit - 1) / kSplit);
+    // The context length and the partials of the first eight splits are requested together (the number
+    // of splits that hold tokens is only needed to mask the values afterwards): one memory round trip
+    // instead of two.  Partials of splits without tokens are whatever the buffer held and are replaced,
+    // never used in arithmetic.
+    const int ctx_raw = ctx_lens[item / n_q_heads];
     const float *base = scratch + (int64_t)item * n_splits * (D + 2);
+    float ms[G], ls[G];
+    float4_t os[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const float *p = base + (int64_t)min(g, n_splits - 1) * (D + 2);
+        ms[g] = p[0];
+        ls[g] = p[1];
+        os[g] = *reinterpret_cast<const float4_t *>(p + 2 + 4 * w4);
+    }
+    const int ctx = min(ctx_raw, max_ctx);
+    const int used = min(n_splits, (ctx + kSplit - 1) / kSplit);
     float m = -INFINITY, l = 0.f;
     float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
     for (int s0 = 0; s0 < used; s0 += G) {
-        float ms[G], ls[G];
-        float4_t os[G];
+        if (s0 > 0) {
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float *p = base + (int64_t)min(s0 + g, n_splits - 1) * (D + 2);
+                ms[g] = p[0];
+                ls[g] = p[1];
+                os[g] = *reinterpret_cast<const float4_t *>(p + 2 + 4 * w4);
+            }
+        }
 #pragma unroll
         for (int g = 0; g < G; g++) {
-            const bool in = s0 + g < used;
-            const float *p = base + (int64_t)(in ? s0 + g : 0) * (D + 2);
-            ms[g] = in ? p[0] : -INFINITY;
-            ls[g] = in ? p[1] : 0.f;
-            os[g] = in ? *reinterpret_cast<const float4_t *>(p + 2 + 4 * w4) : float4_t{0.f, 0.f, 0.f, 0.f};
+            if (s0 + g >= used) {
+                ms[g] = -INFINITY;
+                ls[g] = 0.f;
+                os[g] = float4_t{0.f, 0.f, 0.f, 0.f};
+            }
         }
         float mg = m;
 #pragma unroll

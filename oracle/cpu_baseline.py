@@ -58,7 +58,7 @@ def gemv_baseline(M: int, K: int, mode: str, sample_rows: int, repeats: int = 3,
     f = M / rows
     return {
         "pack_s": t_pack * f, "decode_s": t_dec * f, "compute_s": t_mv * f,
-        "total_s": (t_dec + t_mv) * f,          # pack is an offline step in the reference flow too
+        "total_s": (t_pack + t_dec + t_mv) * f,  # pack, decode and compute are reported separately and summed
         "cores": torch.get_num_threads(), "cpu_count": os.cpu_count(),
         "sample": f"{rows} of {M} rows x {K} cols, {mode}, median of {repeats}; scaled x{f:g}",
     }
@@ -78,13 +78,19 @@ def attention_baseline(heads: int, L: int, d: int, mode: str, sample_heads: int 
     g = torch.Generator().manual_seed(seed)
     lut = torch.from_numpy(dec_table(mode))
     n = min(sample_heads, heads)
-    qkv = [torch.randn(n, L, d, generator=g).half().to(_DT[mode]).view(torch.uint8) for _ in range(3)]
+    src = [torch.randn(n, L, d, generator=g).half() for _ in range(3)]
+    state = {}
+
+    def pack():
+        state["qkv"] = [t.to(_DT[mode]).view(torch.uint8) for t in src]
 
     def run():
         for h in range(n):
-            q, k, v = (lut[t[h].long()] for t in qkv)
+            q, k, v = (lut[t[h].long()] for t in state["qkv"])
             torch.nn.functional.scaled_dot_product_attention(q[None], k[None], v[None])
 
+    t_pack = _median_time(pack, repeats)
     t = _median_time(run, repeats)
-    return {"total_s": t * heads / n, "cores": torch.get_num_threads(),
+    return {"total_s": (t_pack + t) * heads / n, "pack_s": t_pack * heads / n, "compute_s": t * heads / n,
+            "cores": torch.get_num_threads(),
             "sample": f"{n} of {heads} heads, L={L}, d={d}, {mode}; scaled x{heads / n:g}"}

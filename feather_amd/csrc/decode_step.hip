@@ -190,7 +190,8 @@ __global__ __launch_bounds__(kDsThreads) void swiglu_pack_kernel(const float *__
 // written into the paged cache at position pos = ctx_lens[b]; ctx_after[b] = pos + 1.
 // A position outside [0, max_blocks * block_size) or a block id outside [0, n_blocks) is never
 // written: the token is dropped, ctx_after[b] is the old length (clamped into the table) and
-// status[b] says why (1: no room / bad position, 2: bad block id; 0: appended).
+// status[b] says why (1: no room / bad position, 2: bad block id; 0: appended).  pos_limit is the number of
+// positions the caller's context bound allows (at most the table's max_blocks * block_size).
 constexpr int kRopeThreads = 64;
 // sin and cos of a non-negative angle below ~1e5 rad to ~1e-7 absolute: three-constant Cody-Waite reduction
 // by pi/2 with fused multiply-adds, then the single-precision minimax polynomials on [-pi/4, pi/4].  The
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *
                                                                 uint32_t *__restrict__ v_cache,
                                                                 int32_t *__restrict__ ctx_after, int n_blocks,
                                                                 int32_t *__restrict__ status,
-                                                                float *__restrict__ rot_f32) {
+                                                                float *__restrict__ rot_f32, int pos_limit) {
     const int b = blockIdx.x;
     const int dw = d / 4, half_w = d / 8;            // words per head, words per rotation half
     const int heads = n_q + 2 * n_kv;
@@ -241,7 +242,7 @@ __global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *
         pl[u] = *reinterpret_cast<const float4 *>(x + 4 * t + off);            // elements 4t .. 4t+3
         ph[u] = *reinterpret_cast<const float4 *>(x + d / 2 + 4 * t + off);    // their partners
     }
-    const int cap = max_blocks * block_size;
+    const int cap = pos_limit;                       // at most max_blocks * block_size
     const bool pos_ok = pos_raw >= 0 && pos_raw < cap;
     const int pos = pos_ok ? pos_raw : 0;            // in range for the table lookup; nothing is written if !pos_ok
     const int blk = block_tables[(int64_t)b * max_blocks + pos / block_size];
@@ -309,6 +310,105 @@ __global__ __launch_bounds__(kRopeThreads) void rope_append_kernel(const float *
     }
 }
 
+// First kernel of a step when the attention runs with the fused prologue (paged_attn_split_kernel, FUSED):
+// everything that depends only on the step's inputs and is the same for all layers, computed once.
+//   blocks [0, batch)          embedding row of the sequence; the cos / sin pairs of its position (the table the
+//                              rotary embedding of every layer reads); ctx_after and status of the sequence
+//   blocks [batch, batch + n)  one entry of the attention work plan each: the (sequence, split) items in the order
+//                              the attention workgroups take them -- all full 512-token splits in sequence order, then
+//                              the partial last splits by size, largest first -- with the block ids of the split, so
+//                              that an attention workgroup needs one memory round trip to know its work and its blocks
+// A sequence's new token is appended iff its position ctx_lens[b] lies in [0, max_ctx) and the table entry of that
+// position is a block of the cache; otherwise the sequence attends over the tokens it has and status says why.
+constexpr int kPlanSplit = 512;                  // tokens per attention split (paged_attention.hip: kSplit)
+__global__ __launch_bounds__(kDsThreads) void step_prologue_kernel(
+    const _Float16 *__restrict__ embed, const int32_t *__restrict__ tokens, float *__restrict__ h, int hidden,
+    const int32_t *__restrict__ ctx_lens, const int32_t *__restrict__ block_tables, int batch, int d, int block_size,
+    int max_blocks, int n_blocks, int max_ctx, int n_splits, float log2_theta, float *__restrict__ cs,
+    int32_t *__restrict__ plan, int32_t *__restrict__ ctx_after, int32_t *__restrict__ status) {
+    // tokens the sequence holds after the step, whether the new one is appended, and why not
+    auto seq_state = [&](int b, int &total, bool &append, int &why) {
+        const int pos_raw = ctx_lens[b];
+        const bool pos_ok = pos_raw >= 0 && pos_raw < max_ctx;
+        const int blk = block_tables[(int64_t)b * max_blocks + (pos_ok ? pos_raw / block_size : 0)];
+        const bool blk_ok = (unsigned)blk < (unsigned)n_blocks;
+        append = pos_ok && blk_ok;
+        total = append ? pos_raw + 1 : min(max(pos_raw, 0), max_ctx);
+        why = pos_ok ? (blk_ok ? 0 : 2) : 1;
+    };
+    if ((int)blockIdx.x < batch) {
+        const int b = blockIdx.x;
+        int total, why;
+        bool append;
+        seq_state(b, total, append, why);
+        const _Float16 *row = embed + (int64_t)tokens[b] * hidden;
+        for (int i = threadIdx.x; i < hidden; i += kDsThreads) h[(int64_t)b * hidden + i] = (float)row[i];
+        const int pos = append || why == 2 ? ctx_lens[b] : 0;          // a valid position even if the block id is not
+        for (int jj = threadIdx.x; jj < d / 2; jj += kDsThreads) {
+            const float inv_freq = exp2f(-(2.0f * (float)jj / (float)d) * log2_theta);   // as rope_append_kernel
+            float sn, c;
+            sincos_small((float)pos * inv_freq, sn, c);
+            cs[((int64_t)b * (d / 2) + jj) * 2] = c;
+            cs[((int64_t)b * (d / 2) + jj) * 2 + 1] = sn;
+        }
+        if (threadIdx.x == 0) {
+            ctx_after[b] = total;
+            if (status) status[b] = why;
+        }
+        return;
+    }
+    const int item = blockIdx.x - batch, lane = threadIdx.x & 63;
+    const int ids_per = kPlanSplit / block_size;
+    int32_t *entry = plan + (int64_t)item * (4 + ids_per);
+    int total = 0, why = 0;
+    bool append = false;
+    if (lane < batch) seq_state(lane, total, append, why);
+    int seq = -1, split = 0;
+    if (n_splits == 1) {
+        if (item < batch) seq = item;
+    } else {
+        const int nf = total / kPlanSplit, ps = total % kPlanSplit;   // full splits, tokens of the partial one
+        int inc = nf;                                                 // inclusive prefix sum over the lanes
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const int t = __shfl_up(inc, off, kWave);
+            if (lane >= off) inc += t;
+        }
+        const int n_full = __builtin_amdgcn_readlane(inc, kWave - 1);
+        uint64_t hit;
+        if (item < n_full) {
+            const int exc = inc - nf;
+            hit = __builtin_amdgcn_ballot_w64(item >= exc && item < exc + nf);
+            if (hit) split = item - __builtin_amdgcn_readlane(exc, __builtin_ctzll(hit));
+        } else {
+            int rank = 0;                                             // partial splits larger than this lane's (ties: lower sequence first)
+            for (int t = 0; t < batch; t++) {
+                const int pt = __builtin_amdgcn_readlane(ps, t);
+                rank += (pt > ps || (pt == ps && t < lane)) ? 1 : 0;
+            }
+            hit = __builtin_amdgcn_ballot_w64(ps > 0 && rank == item - n_full);
+            if (hit) split = __builtin_amdgcn_readlane(nf, __builtin_ctzll(hit));
+        }
+        if (hit) seq = __builtin_ctzll(hit);
+    }
+    if (seq < 0) {
+        if (threadIdx.x == 0) entry[0] = -1;
+        return;
+    }
+    const int seq_total = __builtin_amdgcn_readlane(total, seq);
+    const bool seq_append = __builtin_amdgcn_readlane((int)append, seq) != 0;
+    if (threadIdx.x == 0) {
+        entry[0] = seq;
+        entry[1] = split;
+        entry[2] = seq_total;
+        entry[3] = seq_append && split == (seq_total - 1) / kPlanSplit ? 1 : 0;   // the new token sits at seq_total - 1
+    }
+    for (int i = threadIdx.x; i < ids_per; i += kDsThreads) {
+        const int bi = split * ids_per + i;
+        entry[4 + i] = bi < max_blocks ? block_tables[(int64_t)seq * max_blocks + bi] : 0;
+    }
+}
+
 // K slices per GEMV: enough 64-row tiles x slices to cover the 256 CUs, at most one slice per
 // 256-column chunk (the launcher's own clamp, repeated here to size the partial buffers)
 static int plan_splits(int64_t M, int64_t K) {
@@ -325,10 +425,11 @@ struct StepPlan {
     int s_qkv, s_o, s_gu, s_down;
     int64_t qkv_rows;
     bool fused_mlp;                              // gate/up GEMV with the SwiGLU epilogue (no fp32 gate/up buffer)
-    size_t b_h, b_delta, b_xq, b_act, b_qkv, b_qp, b_gu, b_ctx;
+    size_t b_h, b_delta, b_xq, b_act, b_qkv, b_qp, b_gu, b_ctx, b_plan, b_cs;
+    bool fused_attn;                             // rotary embedding / query packing / K-V append inside the attention kernel
 };
 
-static StepPlan plan_step(const feather_decoder_t *dec, int64_t batch) {
+static StepPlan plan_step(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx) {
     const int64_t H = dec->hidden, nq = dec->n_q_heads, nkv = dec->n_kv_heads, d = dec->head_dim, I = dec->inter;
     StepPlan P;
     P.qkv_rows = (nq + 2 * nkv) * d;
@@ -346,6 +447,9 @@ static StepPlan plan_step(const feather_decoder_t *dec, int64_t batch) {
     P.b_qp = up(batch * nq * d);
     P.b_gu = P.fused_mlp ? 0 : up((int64_t)P.s_gu * batch * 2 * I * 4);
     P.b_ctx = up(batch * 4);
+    P.fused_attn = paged_attn_fused_supported(batch, nq, nkv, d, dec->block_size, P.s_qkv);
+    P.b_plan = P.fused_attn ? up(paged_attn_plan_ints(batch, dec->block_size, max_ctx) * 4) : 0;
+    P.b_cs = P.fused_attn ? up(batch * (d / 2) * 8) : 0;
     return P;
 }
 
@@ -354,7 +458,7 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
                     const int32_t *ctx_lens, int batch, int max_ctx, void *scratch, float *logits, int32_t *status,
                     hipStream_t s) {
     const int H = dec->hidden, nq = dec->n_q_heads, nkv = dec->n_kv_heads, d = dec->head_dim, I = dec->inter;
-    const StepPlan P = plan_step(dec, batch);
+    const StepPlan P = plan_step(dec, batch, max_ctx);
     const int qkv_rows = (int)P.qkv_rows;
     // scratch carve-up (all offsets multiples of 256 bytes)
     char *p = (char *)scratch;
@@ -367,6 +471,8 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
     uint32_t *qp = (uint32_t *)take(P.b_qp);
     float *gu = (float *)take(P.b_gu);
     int32_t *ctx_after = (int32_t *)take(P.b_ctx);
+    int32_t *plan = (int32_t *)take(P.b_plan);
+    float *cs = (float *)take(P.b_cs);
     void *pa_scratch = p;
     const float scale = 1.0f / sqrtf((float)d);
     const float log2_theta = log2f(dec->rope_theta);
@@ -390,7 +496,14 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
         if (rc != FEATHER_OK) return rc; \
     } while (0)
 
-    hipLaunchKernelGGL(embed_kernel, dim3(batch), dim3(kDsThreads), 0, s, (const _Float16 *)dec->embed_f16, tokens, h, H);
+    if (P.fused_attn) {
+        const int n_splits = max((max_ctx + kPlanSplit - 1) / kPlanSplit, 1);
+        hipLaunchKernelGGL(step_prologue_kernel, dim3(batch + batch * n_splits), dim3(kDsThreads), 0, s,
+                           (const _Float16 *)dec->embed_f16, tokens, h, H, ctx_lens, block_tables, batch, d, dec->block_size,
+                           dec->max_blocks, dec->n_blocks, max_ctx, n_splits, log2_theta, cs, plan, ctx_after, status);
+    } else {
+        hipLaunchKernelGGL(embed_kernel, dim3(batch), dim3(kDsThreads), 0, s, (const _Float16 *)dec->embed_f16, tokens, h, H);
+    }
     DS_CHECK(check_launch("feather_decode_step (embed)"));
     const float *pending = nullptr;                       // output of the previous down projection, not yet added
     const int64_t hs = (int64_t)batch * H;
@@ -399,15 +512,23 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
         launch_norm<MODE>(batch, s, h, pending, P.s_down, hs, L.norm_attn, xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
         DS_CHECK(gemv(L.w_qkv, qkv, qkv_rows, H, P.s_qkv));
-        hipLaunchKernelGGL((rope_append_kernel<MODE>),
-                           dim3(batch, ((nq + 2 * nkv) * (d / 8) + kRopeThreads - 1) / kRopeThreads), dim3(kRopeThreads), 0, s, qkv, ctx_lens,
-                           block_tables, (int64_t)batch * qkv_rows, P.s_qkv, nq, nkv, d, dec->block_size, dec->max_blocks,
-                           log2_theta, qp, (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, ctx_after, dec->n_blocks,
-                           l == 0 ? status : nullptr, (float *)nullptr);
-        DS_CHECK(check_launch("feather_decode_step (rope)"));
-        // attention writes its output already rounded to FP8 and packed (the operand of W_o)
-        DS_CHECK(paged_attn_launch(qp, L.k_cache, L.v_cache, block_tables, ctx_after, nullptr, xq, nullptr, pa_scratch, batch, nq,
-                                   nkv, d, dec->block_size, dec->max_blocks, dec->n_blocks, max_ctx, MODE, scale, s));
+        if (P.fused_attn) {
+            // rotary embedding, query packing and the append of the new K / V rows happen in the attention
+            // kernel's prologue; it writes its output already rounded to FP8 and packed (the operand of W_o)
+            DS_CHECK(paged_attn_fused_launch(plan, ctx_after, L.k_cache, L.v_cache, qkv, P.s_qkv, (int64_t)batch * qkv_rows, cs,
+                                             xq, pa_scratch, batch, nq, nkv, dec->block_size, dec->max_blocks, dec->n_blocks,
+                                             max_ctx, MODE, scale, s));
+        } else {
+            hipLaunchKernelGGL((rope_append_kernel<MODE>),
+                               dim3(batch, ((nq + 2 * nkv) * (d / 8) + kRopeThreads - 1) / kRopeThreads), dim3(kRopeThreads), 0, s, qkv, ctx_lens,
+                               block_tables, (int64_t)batch * qkv_rows, P.s_qkv, nq, nkv, d, dec->block_size, dec->max_blocks,
+                               log2_theta, qp, (uint32_t *)L.k_cache, (uint32_t *)L.v_cache, ctx_after, dec->n_blocks,
+                               l == 0 ? status : nullptr, (float *)nullptr, max_ctx);
+            DS_CHECK(check_launch("feather_decode_step (rope)"));
+            // attention writes its output already rounded to FP8 and packed (the operand of W_o)
+            DS_CHECK(paged_attn_launch(qp, L.k_cache, L.v_cache, block_tables, ctx_after, nullptr, xq, nullptr, pa_scratch, batch, nq,
+                                       nkv, d, dec->block_size, dec->max_blocks, dec->n_blocks, max_ctx, MODE, scale, s));
+        }
         DS_CHECK(gemv(L.w_o, delta, H, nq * d, P.s_o));
         launch_norm<MODE>(batch, s, h, delta, P.s_o, hs, L.norm_mlp, xq, H, dec->rms_eps);
         DS_CHECK(check_launch("feather_decode_step (norm)"));
@@ -431,9 +552,9 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
 }
 
 static int64_t step_scratch_bytes(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx) {
-    const StepPlan P = plan_step(dec, batch);
+    const StepPlan P = plan_step(dec, batch, max_ctx);
     auto up = [](int64_t b) { return (b + 255) / 256 * 256; };
-    return (int64_t)(P.b_h + P.b_delta + P.b_xq + P.b_act + P.b_qkv + P.b_qp + P.b_gu + P.b_ctx) +
+    return (int64_t)(P.b_h + P.b_delta + P.b_xq + P.b_act + P.b_qkv + P.b_qp + P.b_gu + P.b_ctx + P.b_plan + P.b_cs) +
            up(feather_paged_attn_scratch_bytes(batch, dec->n_q_heads, dec->head_dim, max_ctx));
 }
 
@@ -547,7 +668,7 @@ extern "C" int feather_rope_append(const void *qkv_f32, int64_t n_part, int64_t 
                        (const int32_t *)ctx_lens, (const int32_t *)block_tables, part_stride, (int)n_part, (int)n_q_heads, \
                        (int)n_kv_heads, (int)d, (int)block_size, (int)max_blocks, log2f(rope_theta), (uint32_t *)q_packed, \
                        (uint32_t *)k_cache, (uint32_t *)v_cache, (int32_t *)ctx_after, (int)n_blocks, (int32_t *)seq_status, \
-                       (float *)rot_f32)
+                       (float *)rot_f32, (int)(max_blocks * block_size))
     if (mode == FEATHER_E5M2) FEATHER_ROPE(FEATHER_E5M2); else FEATHER_ROPE(FEATHER_E4M3);
 #undef FEATHER_ROPE
     return check_launch(me);

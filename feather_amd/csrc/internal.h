@@ -15,6 +15,19 @@ int paged_attn_launch(const void *q, const void *k_cache, const void *v_cache, c
                       int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size, int64_t max_blocks,
                       int64_t n_blocks, int64_t max_ctx, int mode, float scale, hipStream_t stream);
 
+// The decode step's attention with the rotary embedding, the query packing and the append of the new
+// token's K / V row fused into its prologue (see paged_attn_split_kernel, FUSED).  `plan` and `cs` are
+// written once per step by the step's prologue kernel; plan entries are 4 + 512 / block_size ints:
+// {sequence or -1, split, tokens of the sequence including an appended new one, owner flag, block ids of
+// the split}, one per (sequence, split) item in launch order.  ctx_after [n_seq] is what the merge reads.
+bool paged_attn_fused_supported(int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size,
+                                int64_t n_part);
+int64_t paged_attn_plan_ints(int64_t n_seq, int64_t block_size, int64_t max_ctx);
+int paged_attn_fused_launch(const int32_t *plan, const int32_t *ctx_after, void *k_cache, void *v_cache, const float *qkv,
+                            int n_part, int64_t part_stride, const float *cs, uint32_t *out_packed, void *scratch,
+                            int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads, int64_t block_size, int64_t max_blocks,
+                            int64_t n_blocks, int64_t max_ctx, int mode, float scale, hipStream_t stream);
+
 // Batched GEMV with the K range cut into `splits` slices: slice s writes its partial sums to
 // out_f32 + s * part_stride ([nvec, M] each); the consumer adds the slices in index order.
 // Needs K % 256 == 0 and 16-byte aligned w and x; splits is clamped to K / 256.  Returns the

@@ -75,18 +75,37 @@ __device__ __forceinline__ void v_pairs(uint32_t wa, uint32_t wb, uint32_t out[4
 // (parameter order: what a wave needs before its first loads -- the lengths, the table, the operands
 // and the shape -- fills the 16 dwords of kernel arguments that arrive preloaded in SGPRs; the rest
 // is fetched with s_load while those loads are in flight)
-template <int D, int MODE, bool FAST>
+//
+// FUSED (the decode step's attention; needs FAST and D = 64): the kernel also does what the step otherwise
+// runs as a separate kernel in front of it.  `ctx_lens` then points to the step's work plan (one entry per
+// workgroup item, written once per step: sequence, split, token count, owner flag and the block ids of the
+// split, so that a workgroup knows its work and its blocks after ONE memory round trip), `q` is unused and the
+// query comes from the fused QKV projection's fp32 partial sums `qkv` (n_part slices, part_stride floats
+// apart): the workgroup adds the slices in slice order, applies the rotary embedding with the step's cos / sin
+// table `cs` ([n_seq, D / 2] pairs), rounds to FP8 (quant4) and keeps the packed query heads in LDS.  The
+// workgroup whose split holds the new token's position ("owner") does the same for that token's K and V row of
+// its KV head, appends them to the cache and scores the token from LDS after the cached ones (wave 0, one extra
+// one-token step), so the cached tokens are read from memory and the new one never is.
+constexpr int kFusedMaxPairs = 96;   // (group + 2) * n_part the LDS staging of the FUSED prologue holds
+
+template <int D, int MODE, bool FAST, bool FUSED = false>
 __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     const int32_t *__restrict__ ctx_lens, const int32_t *__restrict__ block_tables, const uint32_t *__restrict__ q,
     const uint32_t *__restrict__ k_cache, const uint32_t *__restrict__ v_cache, int n_q_heads, int n_kv_heads,
     int block_size, int max_blocks, int n_splits, int max_ctx, float scale_log2e, float *__restrict__ scratch,
-    float *__restrict__ out_f32, uint32_t *__restrict__ out_packed, _Float16 *__restrict__ out_q16, uint32_t max_blk) {
+    float *__restrict__ out_f32, uint32_t *__restrict__ out_packed, _Float16 *__restrict__ out_q16, uint32_t max_blk,
+    const float *__restrict__ qkv, int n_part, int64_t part_stride, const float *__restrict__ cs,
+    uint32_t *__restrict__ k_cache_w, uint32_t *__restrict__ v_cache_w) {
+    static_assert(!FUSED || (FAST && D == 64), "the fused prologue is written for D = 64 and power-of-two blocks");
     const int bs_shift = FAST ? __builtin_ctz((unsigned)block_size) : 0;
     constexpr int DW = D / 4;       // words per token row
     constexpr int RB = D / 64;      // 16-word row blocks of V per token
     constexpr int STEPS = D / 32;   // MFMA k-steps of the score product
     __shared__ float ml_lds[kPaWaves][2][16];
     __shared__ float4_t o_lds[kPaWaves - 1][RB * 4][kWave];
+    __shared__ float4_t part_lds[FUSED ? kFusedMaxPairs * (D / 8) * 2 : 1];   // [slice][head slot][D/8 threads][lo, hi]
+    __shared__ uint32_t q_lds[FUSED ? 16 * DW : 1];                             // packed query heads of the group
+    __shared__ uint32_t kv_new[FUSED ? 2 * DW : 1];                             // packed K and V row of the new token
 
     // Work item of this workgroup.  With one split per sequence the grid is exactly the
     // (sequence, KV head) pairs.  Otherwise the grid is sized for max_ctx and most sequences use
@@ -100,7 +119,18 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     const int kvh = blockIdx.x % n_kv_heads;
     int seq = blockIdx.x / n_kv_heads, split = 0;
     int ctx_raw;
-    if (n_splits > 1) {
+    bool owner = false;                                     // FUSED: this workgroup appends and scores the new token
+    const int32_t *entry = nullptr;
+    if constexpr (FUSED) {
+        // plan entry: {sequence (-1: no work), split, tokens of the sequence incl. the new one, owner flag, block ids of the split}
+        // (an entry without work has sequence -1; the test waits until the block ids of the entry have been
+        // requested, so that header and ids arrive in one round trip: every entry has all its id slots)
+        entry = ctx_lens + (int64_t)(blockIdx.x / n_kv_heads) * (4 + (kSplit >> bs_shift));
+        seq = entry[0];
+        split = entry[1];
+        ctx_raw = entry[2];
+        owner = entry[3] != 0;
+    } else if (n_splits > 1) {
         const int n_seq = gridDim.x / (n_splits * n_kv_heads);
         const int item = blockIdx.x / n_kv_heads;          // index over the (sequence, split) pairs that exist
         seq = -1;
@@ -178,9 +208,10 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
 #pragma unroll
     for (int st = 0; st < STEPS; st++) {
         qw[st] = u32x2{0, 0};
-        if (j < group)
-            qw[st] = *reinterpret_cast<const u32x2 *>(q + (int64_t)(seq * n_q_heads + qh) * DW + 16 * (st / 2) + 4 * kb +
-                                                      2 * (st % 2));
+        if constexpr (!FUSED)
+            if (j < group)
+                qw[st] = *reinterpret_cast<const u32x2 *>(q + (int64_t)(seq * n_q_heads + qh) * DW + 16 * (st / 2) +
+                                                          4 * kb + 2 * (st % 2));
     }
 
     // One step = packed K (16 codes of the lane's token per 64-dim chunk) and V (word j of 8 tokens).
@@ -201,17 +232,24 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
     auto fetch_ids = [&](Step &T, int t0) {
 #pragma unroll
         for (int a = 0; a < 2; a++) {
-            T.kid[a] = bt[blk_of(min(t0 + 16 * a + j, t_cap))];
+            if constexpr (FUSED) {                // the split's ids sit in the plan entry (every slot of it is filled)
+                T.kid[a] = entry[4 + ((t0 - t_begin + 16 * a + j) >> bs_shift)];
+                T.vid[a][0] = entry[4 + ((t0 - t_begin + 16 * a + 4 * kb) >> bs_shift)];
+            } else {
+                T.kid[a] = bt[blk_of(min(t0 + 16 * a + j, t_cap))];
 #pragma unroll
-            for (int r = 0; r < (FAST ? 1 : 4); r++) T.vid[a][r] = bt[blk_of(min(t0 + 16 * a + 4 * kb + r, t_cap))];
+                for (int r = 0; r < (FAST ? 1 : 4); r++) T.vid[a][r] = bt[blk_of(min(t0 + 16 * a + 4 * kb + r, t_cap))];
+            }
         }
     };
     int fallback = 0;                             // block of the split's first token: valid whenever the split has work
     if (max_ctx > 0) {
-        fallback = bt[blk_of(min(t_begin, t_cap))];
+        fallback = FUSED ? entry[4] : bt[blk_of(min(t_begin, t_cap))];
 #pragma unroll
         for (int f = 0; f < NF; f++) fetch_ids(steps[f], t_begin + kStepTok * (wave + kPaWaves * f));
     }
+    if constexpr (FUSED)
+        if (seq < 0) return;                      // beyond the last item (whole workgroup)
 
     const int ctx = min(ctx_raw, max_ctx);        // never index past the block table
     if (t_begin >= ctx) {                         // empty split: the merge never reads it
@@ -225,12 +263,15 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         }
         return;
     }
-    const int t_end = min(t_begin + kSplit, ctx);
+    // tokens of this split that are read from the cache: the owner's new token (position ctx - 1) is not among them
+    const int t_end = min(t_begin + kSplit, owner ? ctx - 1 : ctx);
     const int n_steps = (t_end - t_begin + kStepTok - 1) / kStepTok;
 
     half8_t qf[STEPS];
+    if constexpr (!FUSED) {
 #pragma unroll
-    for (int st = 0; st < STEPS; st++) qf[st] = pa_dec8<MODE>(qw[st].x, qw[st].y);
+        for (int st = 0; st < STEPS; st++) qf[st] = pa_dec8<MODE>(qw[st].x, qw[st].y);
+    }
 
     float4_t o[RB][4];
 #pragma unroll
@@ -249,27 +290,27 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         return (int64_t)(uint32_t)((min((uint32_t)blk, max_blk) * n_kv_heads + kvh) * block_size + slot_of(tok));
     };
     auto load_step = [&](Step &S, int t0) {
-        const bool full = t0 + kStepTok <= ctx;   // wave-uniform: every token of the step exists
+        const bool full = t0 + kStepTok <= t_end; // wave-uniform: every token of the step exists
 #pragma unroll
         for (int a = 0; a < 2; a++) {
             const int tk = t0 + 16 * a + j;
-            const uint32_t *kr = k_cache + row_base(full || tk < ctx ? S.kid[a] : fallback, tk) * DW;
+            const uint32_t *kr = k_cache + row_base(full || tk < t_end ? S.kid[a] : fallback, tk) * DW;
 #pragma unroll
             for (int c64 = 0; c64 < RB; c64++) S.kw[a][c64] = *reinterpret_cast<const u32x4 *>(kr + 16 * c64 + 4 * kb);
             const int tq = t0 + 16 * a + 4 * kb;
             const uint32_t *vq = nullptr;
             if constexpr (FAST)                   // an aligned group of 4 tokens shares a block
-                vq = v_cache + row_base(full || tq < ctx ? S.vid[a][0] : fallback, tq) * DW + j;
+                vq = v_cache + row_base(full || tq < t_end ? S.vid[a][0] : fallback, tq) * DW + j;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const uint32_t *vr = vq + r * DW;
-                if constexpr (!FAST) vr = v_cache + row_base(full || tq + r < ctx ? S.vid[a][r] : fallback, tq + r) * DW + j;
+                if constexpr (!FAST) vr = v_cache + row_base(full || tq + r < t_end ? S.vid[a][r] : fallback, tq + r) * DW + j;
                 if (full) {
 #pragma unroll
                     for (int rb = 0; rb < RB; rb++) S.vw[rb][a][r] = vr[16 * rb];
                 } else {
 #pragma unroll
-                    for (int rb = 0; rb < RB; rb++) S.vw[rb][a][r] = tq + r < ctx ? vr[16 * rb] : 0u;
+                    for (int rb = 0; rb < RB; rb++) S.vw[rb][a][r] = tq + r < t_end ? vr[16 * rb] : 0u;
                 }
             }
         }
@@ -340,9 +381,94 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         }
     };
 
+    float4_t cs01 = float4_t{0.f, 0.f, 0.f, 0.f}, cs23 = cs01;     // FUSED: (cos, sin) of this thread's four element pairs
+    if constexpr (FUSED) {
+        // ---- query (and, for the owner, the new token's K / V row) from the QKV projection's partial sums.
+        // Phase A: every (slice, head slot, 4 + 4 elements) unit is fetched by some thread -- spread over the
+        // whole workgroup so that a thread holds two or three units, not every slice of its element -- and
+        // parked in LDS; the cos / sin pairs of the threads that will rotate are fetched in the same round.
+        constexpr int T8 = D / 8;                                  // threads per head slot: 4 low + 4 high elements each
+        const int heads = n_q_heads + 2 * n_kv_heads;
+        const int slots = group + (owner ? 2 : 0);                 // query heads of the group, then the K and the V head
+        const int units = n_part * slots * T8;
+        auto src_row = [&](int slot) {
+            return slot < group ? kvh * group + slot : (slot == group ? n_q_heads + kvh : n_q_heads + n_kv_heads + kvh);
+        };
+        constexpr int kUnitsPerThread = (kFusedMaxPairs * T8 + kPaThreads - 1) / kPaThreads;
+        float4_t plo[kUnitsPerThread], phi[kUnitsPerThread];
+#pragma unroll
+        for (int it = 0; it < kUnitsPerThread; it++) {
+            const int u = min((int)threadIdx.x + it * kPaThreads, units - 1);   // surplus threads repeat the last unit
+            const int tt = u % T8, slot = (u / T8) % slots, slice = u / (T8 * slots);
+            const float *x = qkv + ((int64_t)seq * heads + src_row(slot)) * D + (int64_t)slice * part_stride;
+            plo[it] = *reinterpret_cast<const float4_t *>(x + 4 * tt);
+            phi[it] = *reinterpret_cast<const float4_t *>(x + D / 2 + 4 * tt);
+        }
+        const int my_tt = threadIdx.x % T8;
+        const float4_t *csp = reinterpret_cast<const float4_t *>(cs + ((int64_t)seq * (D / 2) + 4 * my_tt) * 2);
+        cs01 = csp[0];                                             // (cos, sin) of elements 4 tt .. 4 tt + 3
+        cs23 = csp[1];
+#pragma unroll
+        for (int it = 0; it < kUnitsPerThread; it++) {
+            const int u = threadIdx.x + it * kPaThreads;
+            if (u < units) {
+                part_lds[2 * u] = plo[it];
+                part_lds[2 * u + 1] = phi[it];
+            }
+        }
+    }
+    // Phase B runs inside the first turn of the main loop, behind the loads of the wave's first steps: the cached
+    // K / V rows are in flight while the query is rotated and packed.  (The partial sums are parked in LDS before
+    // those loads go out: issued the other way round, the 64 destination registers of the rows would be live
+    // together with the partial sums' and one workgroup less would fit a CU.)
+    auto fused_phase_b = [&]() {
+        constexpr int T8 = D / 8;
+        const int slots = group + (owner ? 2 : 0);
+        const bool rotates = (int)threadIdx.x < slots * T8;
+        const int my_slot = rotates ? threadIdx.x / T8 : 0, my_tt = threadIdx.x % T8;
+        __syncthreads();
+        // Phase B: one thread per (head slot, 4 + 4 elements) adds the slices in slice order, rotates (query and
+        // K heads), rounds to FP8 and packs: the arithmetic of the stand-alone rotary kernel, value for value.
+        if (rotates) {
+            float4_t lo = part_lds[2 * (my_slot * T8 + my_tt)], hi = part_lds[2 * (my_slot * T8 + my_tt) + 1];
+            for (int sl = 1; sl < n_part; sl++) {
+                lo += part_lds[2 * ((sl * slots + my_slot) * T8 + my_tt)];
+                hi += part_lds[2 * ((sl * slots + my_slot) * T8 + my_tt) + 1];
+            }
+            if (my_slot <= group) {                                // query heads and the K head; V is not rotated
+                const float c4[4] = {cs01[0], cs01[2], cs23[0], cs23[2]}, s4[4] = {cs01[1], cs01[3], cs23[1], cs23[3]};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float a = lo[i], bb = hi[i];
+                    lo[i] = a * c4[i] - bb * s4[i];
+                    hi[i] = bb * c4[i] + a * s4[i];
+                }
+            }
+            const uint32_t wlo = quant4<MODE>(lo[0], lo[1], lo[2], lo[3]), whi = quant4<MODE>(hi[0], hi[1], hi[2], hi[3]);
+            if (my_slot < group) {
+                q_lds[my_slot * DW + my_tt] = wlo;
+                q_lds[my_slot * DW + my_tt + T8] = whi;
+            } else {                                               // owner only: append the row and keep it for the extra step
+                const int which = my_slot - group, pos = ctx - 1;
+                kv_new[which * DW + my_tt] = wlo;
+                kv_new[which * DW + my_tt + T8] = whi;
+                uint32_t *row = (which ? v_cache_w : k_cache_w) + row_base(entry[4 + ((pos - t_begin) >> bs_shift)], pos) * DW;
+                row[my_tt] = wlo;
+                row[my_tt + T8] = whi;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int st = 0; st < STEPS; st++) {
+            if (j < group) qw[st] = *reinterpret_cast<const u32x2 *>(&q_lds[j * DW + 16 * (st / 2) + 4 * kb + 2 * (st % 2)]);
+            qf[st] = pa_dec8<MODE>(qw[st].x, qw[st].y);
+        }
+    };
+
     // The wave's steps are wave, wave + 4, ...; NF of them are in flight together: a wave has only
-    // a handful of steps, so their chains must overlap each other.
-    for (int st = wave; st < n_steps; st += kPaWaves * NF) {
+    // a handful of steps, so their chains must overlap each other.  (FUSED: every wave makes the first turn,
+    // also one without steps, because that turn holds the workgroup barriers of the query's phase B.)
+    for (int st = wave; st < n_steps || (FUSED && st == wave); st += kPaWaves * NF) {
         if (st != wave) {
 #pragma unroll
             for (int f = 0; f < NF; f++)
@@ -351,9 +477,47 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
 #pragma unroll
         for (int f = 0; f < NF; f++)
             if (st + kPaWaves * f < n_steps) load_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
+        if constexpr (FUSED)
+            if (st == wave) fused_phase_b();
 #pragma unroll
         for (int f = 0; f < NF; f++)
             if (st + kPaWaves * f < n_steps) compute_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
+    }
+
+    if constexpr (FUSED) {
+        // ---- the new token, scored from LDS by wave 0 of its owner as one more step of one token
+        if (owner && wave == 0) {
+            float sc = 0.f;
+#pragma unroll
+            for (int st = 0; st < STEPS; st++) {
+                const u32x2 kw = *reinterpret_cast<const u32x2 *>(&kv_new[16 * (st / 2) + 4 * kb + 2 * (st % 2)]);
+                const u32x4 kd = __builtin_bit_cast(u32x4, pa_dec8<MODE>(kw.x, kw.y)), qd = __builtin_bit_cast(u32x4, qf[st]);
+                sc = dot2(kd.x, qd.x, sc);
+                sc = dot2(kd.y, qd.y, sc);
+                sc = dot2(kd.z, qd.z, sc);
+                sc = dot2(kd.w, qd.w, sc);
+            }
+            sc += __shfl_xor(sc, 16, kWave);                       // the four lanes of a head hold a quarter of the dims each
+            sc += __shfl_xor(sc, 32, kWave);
+            const float m_new = max_raw(m_run, sc * scale_log2e);
+            const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sc, scale_log2e, -m_new));
+            const float pf = (float)(_Float16)e;                   // P is rounded to fp16 before it multiplies V
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+            l_run = l_run * alpha + (kb == 0 ? e : 0.f);           // the lanes' sums are added over kb at the end
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    // accumulator row 4 kb + r of block c is head dim 64 rb + 4 (4 kb + r) + c: word 16 rb + 4 kb + r, byte c
+                    const u32x2 vd = dequant4<MODE>(kv_new[DW + 16 * rb + 4 * kb + r]);
+                    const half2_t v01 = as_half2(vd.x), v23 = as_half2(vd.y);
+                    o[rb][0][r] = o[rb][0][r] * alpha + pf * (float)v01.x;
+                    o[rb][1][r] = o[rb][1][r] * alpha + pf * (float)v01.y;
+                    o[rb][2][r] = o[rb][2][r] * alpha + pf * (float)v23.x;
+                    o[rb][3][r] = o[rb][3][r] * alpha + pf * (float)v23.y;
+                }
+        }
     }
 
     // ---- merge the four waves through LDS (wave 0 finishes)
@@ -513,12 +677,14 @@ static int launch_paged(const void *q, const void *kc, const void *vc, const voi
         hipLaunchKernelGGL((paged_attn_split_kernel<D, MODE, true>), dim3((unsigned)blocks), dim3(kPaThreads), 0, s,
                            (const int32_t *)cl, (const int32_t *)bt, (const uint32_t *)q, (const uint32_t *)kc,
                            (const uint32_t *)vc, (int)n_q_heads, (int)n_kv_heads, (int)block_size, (int)max_blocks, n_splits,
-                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16, (uint32_t)(n_blocks - 1));
+                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16, (uint32_t)(n_blocks - 1),
+                           (const float *)nullptr, 0, (int64_t)0, (const float *)nullptr, (uint32_t *)nullptr, (uint32_t *)nullptr);
     else
         hipLaunchKernelGGL((paged_attn_split_kernel<D, MODE, false>), dim3((unsigned)blocks), dim3(kPaThreads), 0, s,
                            (const int32_t *)cl, (const int32_t *)bt, (const uint32_t *)q, (const uint32_t *)kc,
                            (const uint32_t *)vc, (int)n_q_heads, (int)n_kv_heads, (int)block_size, (int)max_blocks, n_splits,
-                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16, (uint32_t)(n_blocks - 1));
+                           (int)max_ctx, scale * log2e, (float *)scratch, out_f32, out_packed, out_q16, (uint32_t)(n_blocks - 1),
+                           (const float *)nullptr, 0, (int64_t)0, (const float *)nullptr, (uint32_t *)nullptr, (uint32_t *)nullptr);
     int rc = check_launch("feather_paged_attn_fp8");
     if (rc != FEATHER_OK || n_splits == 1) return rc;
     int64_t threads = n_seq * n_q_heads * (D / 4);
@@ -526,6 +692,49 @@ static int launch_paged(const void *q, const void *kc, const void *vc, const voi
                        (const float *)scratch, (const int32_t *)cl, out_f32, out_packed, out_q16, (int)(n_seq * n_q_heads),
                        (int)n_q_heads, n_splits, (int)max_ctx);
     return check_launch("feather_paged_attn_fp8 (merge)");
+}
+
+bool paged_attn_fused_supported(int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads, int64_t d, int64_t block_size,
+                                int64_t n_part) {
+    bool pow2 = block_size >= 4 && block_size <= kSplit && (block_size & (block_size - 1)) == 0;
+    return d == 64 && pow2 && n_seq <= kWave && n_part >= 1 &&
+           (n_q_heads / n_kv_heads + 2) * n_part <= kFusedMaxPairs;
+}
+
+int64_t paged_attn_plan_ints(int64_t n_seq, int64_t block_size, int64_t max_ctx) {
+    int64_t n_splits = (max_ctx + kSplit - 1) / kSplit;
+    if (n_splits < 1) n_splits = 1;
+    return n_seq * n_splits * (4 + kSplit / block_size);
+}
+
+int paged_attn_fused_launch(const int32_t *plan, const int32_t *ctx_after, void *k_cache, void *v_cache, const float *qkv,
+                            int n_part, int64_t part_stride, const float *cs, uint32_t *out_packed, void *scratch,
+                            int64_t n_seq, int64_t n_q_heads, int64_t n_kv_heads, int64_t block_size, int64_t max_blocks,
+                            int64_t n_blocks, int64_t max_ctx, int mode, float scale, hipStream_t s) {
+    int n_splits = (int)((max_ctx + kSplit - 1) / kSplit);
+    if (n_splits < 1) n_splits = 1;
+    const int64_t blocks = n_seq * n_kv_heads * n_splits;
+    FEATHER_CHECK(blocks < (1ll << 31), FEATHER_ESHAPE, "feather_decode_step: attention grid too large");
+    const float log2e = 1.4426950408889634f;
+#define FEATHER_PAF(MM)                                                                                                \
+    hipLaunchKernelGGL((paged_attn_split_kernel<64, MM, true, true>), dim3((unsigned)blocks), dim3(kPaThreads), 0, s, plan, \
+                       (const int32_t *)nullptr, (const uint32_t *)nullptr, (const uint32_t *)k_cache,                 \
+                       (const uint32_t *)v_cache, (int)n_q_heads, (int)n_kv_heads, (int)block_size, (int)max_blocks,   \
+                       n_splits, (int)max_ctx, scale * log2e, (float *)scratch, (float *)nullptr, out_packed,         \
+                       (_Float16 *)nullptr, (uint32_t)(n_blocks - 1), qkv, n_part, part_stride, cs, (uint32_t *)k_cache, \
+                       (uint32_t *)v_cache)
+    if (mode == FEATHER_E5M2) FEATHER_PAF(FEATHER_E5M2); else FEATHER_PAF(FEATHER_E4M3);
+#undef FEATHER_PAF
+    int rc = check_launch("feather_decode_step (attention)");
+    if (rc != FEATHER_OK || n_splits == 1) return rc;
+    const int64_t threads = n_seq * n_q_heads * (64 / 4);
+#define FEATHER_PAM(MM)                                                                                                \
+    hipLaunchKernelGGL((paged_attn_merge_kernel<64, MM>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,   \
+                       (const float *)scratch, ctx_after, (float *)nullptr, out_packed, (_Float16 *)nullptr,          \
+                       (int)(n_seq * n_q_heads), (int)n_q_heads, n_splits, (int)max_ctx)
+    if (mode == FEATHER_E5M2) FEATHER_PAM(FEATHER_E5M2); else FEATHER_PAM(FEATHER_E4M3);
+#undef FEATHER_PAM
+    return check_launch("feather_decode_step (attention merge)");
 }
 
 int paged_attn_launch(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,

@@ -49,14 +49,16 @@ def rope(x: np.ndarray, pos: int, theta: float) -> np.ndarray:
 
 
 def online_attention(dots: np.ndarray, V: np.ndarray, scale: float, chunk: int = 32, split: int = 512,
-                     waves: int = 4) -> np.ndarray:
+                     waves: int = 4, new_token_separate: bool = False) -> np.ndarray:
     """Single-query attention with the evaluation order of csrc/paged_attention.hip: tokens in
     splits of 512; the 32-token chunks of a split are dealt round robin to 4 waves, each of which
     keeps a running maximum (log2 domain), rounds P to fp16 relative to it for P.V, sums the
     denominator from the unrounded P and rescales O when the maximum moves; the waves of a
     split, then the splits, are merged by their maxima.  (Rounding P relative to a running
     instead of the global maximum moves results by ~2^-12, which is enough to flip an FP8 code
-    downstream, hence the same order here.)"""
+    downstream, hence the same order here.)  With new_token_separate the last token is not part of the
+    chunks: wave 0 of the split that holds it takes it as one more chunk of one token after its own chunks,
+    which is how the decode step's attention scores the token it has just appended."""
     c = np.float32(scale * 1.4426950408889634)
     x = (dots.astype(np.float32) * c).astype(np.float32)
     n, d = V.shape
@@ -71,18 +73,26 @@ def online_attention(dots: np.ndarray, V: np.ndarray, scale: float, chunk: int =
             den = np.float32(den + w * l)
         return mg, den, num
 
+    n_chunked = n - 1 if new_token_separate else n
     split_parts = []
     for s0 in range(0, n, split):
-        s1 = min(s0 + split, n)
+        s1 = min(s0 + split, n_chunked)
         wave_parts = []
         for w in range(waves):
             m, l, o = -np.inf, np.float32(0), np.zeros(d, dtype=np.float64)
-            for c0 in range(s0 + w * chunk, s1, waves * chunk):
-                xs = x[c0:min(c0 + chunk, s1)]
+            starts = list(range(s0 + w * chunk, s1, waves * chunk))
+            if new_token_separate and w == 0 and s0 <= n - 1 < s0 + split:
+                starts.append(n - 1)                                  # the new token: one more chunk of one token
+            for c0 in starts:
+                if c0 == n - 1 and new_token_separate:
+                    s1_ = n
+                else:
+                    s1_ = s1
+                xs = x[c0:min(c0 + chunk, s1_)]
                 m_new = max(m, float(xs.max()))
                 alpha = np.float32(np.exp2(np.float32(m - m_new))) if np.isfinite(m) else np.float32(0)
                 # the kernel evaluates 2^(s * c - m) with one fused multiply-add per score
-                raw = dots[c0:min(c0 + chunk, s1)].astype(np.float32).astype(np.float64)
+                raw = dots[c0:min(c0 + chunk, s1_)].astype(np.float32).astype(np.float64)
                 p = np.exp2((raw * float(c) - m_new).astype(np.float32)).astype(np.float32)
                 l = np.float32(l * alpha + p.sum(dtype=np.float32))
                 o = o * float(alpha) + p.astype(np.float16).astype(np.float64) @ V[c0:c0 + len(xs)]
@@ -93,11 +103,14 @@ def online_attention(dots: np.ndarray, V: np.ndarray, scale: float, chunk: int =
     return (num / float(den)).astype(np.float32)
 
 
-def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables, ctx_lens, mode):
+def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables, ctx_lens, mode,
+                    new_token_separate: bool = True):
     """weights: fp16 numpy arrays under the names of PackedDecoder; k_caches / v_caches: per-layer
     uint32 arrays [n_blocks, n_kv, block_size, d/4], updated in place.  Returns logits [B, vocab] float32.
     mode None runs the same composition without any FP8 rounding on float caches
-    [n_blocks, n_kv, block_size, d] (used to pin the composition against library routines)."""
+    [n_blocks, n_kv, block_size, d] (used to pin the composition against library routines).
+    new_token_separate: evaluation order of the attention (see online_attention): True for the step's
+    fused attention kernel (head dim 64, power-of-two blocks), False for its generic path."""
     store = (lambda a: quant_codes(a, mode)) if mode is not None else (lambda a: np.asarray(a, dtype=np.float32))
     load = (lambda w_, n_, d_: decode_np(w_, mode).reshape(n_, d_)) if mode is not None else \
         (lambda w_, n_, d_: np.asarray(w_, dtype=np.float64).reshape(n_, d_))
@@ -130,7 +143,8 @@ def decode_step_ref(cfg, weights: dict, k_caches, v_caches, tokens, block_tables
                 Kd = load(k_caches[l][blocks, kvh, slots], n, d)
                 Vd = load(v_caches[l][blocks, kvh, slots], n, d)
                 for hq in range(kvh * (nq // nkv), (kvh + 1) * (nq // nkv)):     # query head hq reads KV head hq // group
-                    attn[b, hq * d:(hq + 1) * d] = online_attention(Kd @ qd[hq], Vd, float(scale))
+                    attn[b, hq * d:(hq + 1) * d] = online_attention(Kd @ qd[hq], Vd, float(scale),
+                                                                      new_token_separate=new_token_separate)
         o = (quant(attn, mode) @ Wq(g("wo")).T).astype(np.float32)
         h = h + o
         xq = quant(rmsnorm(h, g("norm_mlp"), cfg.rms_eps), mode)

@@ -42,13 +42,17 @@ def _assert_untouched_elsewhere(got: np.ndarray, before: np.ndarray, bt, ctx, bs
     assert np.array_equal(got[mask], before[mask]), f"{what}: a cache row outside the appended slots changed"
 
 
-@pytest.mark.parametrize("mode,hidden,nq,nkv,inter", [("E4M3", 512, 8, 2, 1024), ("E5M2", 256, 4, 4, 512),
-                                                      ("E4M3", 1024, 16, 1, 1536), ("E4M3", 320, 5, 1, 704)])
-def test_decode_step_vs_oracle(orc, mode, hidden, nq, nkv, inter):
+@pytest.mark.parametrize("mode,hidden,nq,nkv,inter,block", [
+    ("E4M3", 512, 8, 2, 1024, 16), ("E5M2", 256, 4, 4, 512, 16), ("E4M3", 1024, 16, 1, 1536, 16), ("E4M3", 320, 5, 1, 704, 16),
+    # a block size that is not a power of two: the step runs the stand-alone rotary kernel and the generic attention
+    ("E4M3", 512, 8, 2, 1024, 12), ("E5M2", 256, 4, 2, 512, 8)])
+def test_decode_step_vs_oracle(orc, mode, hidden, nq, nkv, inter, block):
     from feather_amd.routines.decode import DecoderConfig, PackedDecoder, random_weights
     from oracle import decode_ref
     dev = torch.device("cuda:0")
-    cfg = DecoderConfig(n_layers=2, hidden=hidden, n_q_heads=nq, n_kv_heads=nkv, head_dim=64, inter=inter, vocab=1000)
+    cfg = DecoderConfig(n_layers=2, hidden=hidden, n_q_heads=nq, n_kv_heads=nkv, head_dim=64, inter=inter, vocab=1000,
+                        block_size=block)
+    fused = block & (block - 1) == 0                           # the attention kernel with the fused rotary prologue
     B, max_blocks = 3, 6
     n_blocks = B * max_blocks + 2
     w = random_weights(cfg, seed=hidden)
@@ -74,7 +78,8 @@ def test_decode_step_vs_oracle(orc, mode, hidden, nq, nkv, inter):
         status = torch.full((B,), -1, dtype=torch.int32, device=dev)
         logits = dec.step(tokens.to(dev), bt.to(dev), ctx.to(dev), status=status).cpu().numpy()
         assert status.cpu().tolist() == [0] * B
-        want = decode_ref.decode_step_ref(cfg, wnp, kc_np, vc_np, tokens.numpy(), bt.numpy(), ctx.numpy(), mode)
+        want = decode_ref.decode_step_ref(cfg, wnp, kc_np, vc_np, tokens.numpy(), bt.numpy(), ctx.numpy(), mode,
+                                          new_token_separate=fused)
         err = np.abs(logits - want).max() / np.abs(want).max()
         assert err <= 2e-2, f"step {step}: normalised logit error {err}"
         assert np.mean(np.abs(logits - want) <= 2e-3 * np.abs(want).max()) >= 0.97

@@ -103,9 +103,15 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMV workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--prewarm", type=int, default=1200,
+                    help="untimed launches of the headline kernel that bring the clocks up before the warm-up steps "
+                         "(counter runs under rocprofv3 --pmc use a small number: counters do not depend on the clock)")
+    ap.add_argument("--warm-ms", type=float, default=WARM_MS,
+                    help="milliseconds of back-to-back warm-up calls before each attention / decode series")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (known traffic) to scale rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
+    warm_ms = args.warm_ms
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (every routine is single-device); --gpus must be 1",
               file=sys.stderr)
@@ -146,7 +152,7 @@ def main() -> int:
     # Clock ramp: the first tens of milliseconds of GPU work in a process run below the sustained clock
     # (three back-to-back series of 200 launches measured 45.7, 43.9 and 43.0 us), so the same launches
     # run for ~50 ms before the W warm-up steps; the timed region stays exactly K steps.
-    PREWARM = 1200
+    PREWARM = args.prewarm
     sync()
     cold_us = gpu_time_us(gemv_step("E4M3"), args.steps, 0, sync)   # the first series of the process, no warm-up at all
     for i in range(PREWARM):
@@ -266,25 +272,25 @@ def main() -> int:
             qkv16 = [randn(B, H, L, d).half() for _ in range(3)]
             pk = [feather.pack_fp8_tensor(t, mode="E5M2").view(B, H, L, d // 4) for t in qkv16]
             us = gpu_time_us(lambda i: feather.flash_attention_fp8_e5m2_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4),
-                             10, 10, sync, WARM_MS)
+                             10, 10, sync, warm_ms)
             flops = 4.0 * B * H * L * L * d
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / us / 1e6, 1)
             extra[f"flash_attn_e5m2_b4h16_d64_L{L}_mfma_frac"] = round(flops / us / 1e6 / MFMA_PEAK_F16_TFLOPS, 4)
-            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync, WARM_MS)
+            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync, warm_ms)
             extra[f"sdpa_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
             if L == 8192:   # causal prefill (half the flops) vs causal fp16 SDPA
                 us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
-                                                                                    mode="E5M2", causal=True), 10, 10, sync, WARM_MS)
+                                                                                    mode="E5M2", causal=True), 10, 10, sync, warm_ms)
                 extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
                 extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / 2 / us / 1e6, 1)
                 us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16, is_causal=True),
-                                      10, 10, sync, WARM_MS)
+                                      10, 10, sync, warm_ms)
                 extra[f"sdpa_causal_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
             if L == 8192:   # the same shape with E4M3 codes (fp16 score product: the E4M3 kernel decode is not the matrix core's format)
                 pk4 = [feather.pack_fp8_tensor(t, mode="E4M3").view(B, H, L, d // 4) for t in qkv16]
                 us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk4[0], pk4[1], pk4[2], L, d // 4, mode="E4M3"),
-                                 10, 10, sync, WARM_MS)
+                                 10, 10, sync, warm_ms)
                 extra[f"flash_attn_e4m3_b4h16_d64_L{L}_us"] = round(us, 1)
                 extra[f"flash_attn_e4m3_b4h16_d64_L{L}_TFLOPs"] = round(flops / us / 1e6, 1)
                 del pk4
@@ -295,10 +301,10 @@ def main() -> int:
             qkv16 = [randn(B, H, L, d).half() for _ in range(3)]
             pk = [feather.pack_fp8_tensor(t, mode="E4M3").view(B, H, L, d // 4) for t in qkv16]
             us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
-                                                                                mode="E4M3"), 10, 10, sync, WARM_MS)
+                                                                                mode="E4M3"), 10, 10, sync, warm_ms)
             extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_us"] = round(us, 1)
             extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_TFLOPs"] = round(4.0 * B * H * L * L * d / us / 1e6, 1)
-            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync, WARM_MS)
+            us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync, warm_ms)
             extra[f"sdpa_fp16_b1h8_d{d}_L{L}_us"] = round(us_sdpa, 1)
             del qkv16, pk
         torch.cuda.empty_cache()
@@ -347,7 +353,7 @@ def main() -> int:
             cl = torch.randint(512, cmax, (batch,), generator=g, device=dev, dtype=torch.int32)
             tok = torch.randint(0, cfg.vocab, (batch,), generator=g, device=dev, dtype=torch.int32)
             logits = torch.empty((batch, cfg.vocab), dtype=torch.float32, device=dev)
-            us = gpu_time_us(lambda i: dec.step(tok, btd, cl, out=logits), 20, 10, sync, WARM_MS)
+            us = gpu_time_us(lambda i: dec.step(tok, btd, cl, out=logits), 20, 10, sync, warm_ms)
             step_bytes = dec.weight_bytes() + int(cl.sum().item()) * 2 * cfg.n_kv_heads * cfg.head_dim * cfg.n_layers
             key = f"decode_tinyllama_b{batch}_{mode.lower()}"
             extra[key + "_ms_per_step"] = round(us / 1e3, 3)

@@ -18,8 +18,8 @@
 namespace feather {
 
 constexpr int kDotThreads = 256;
-constexpr int kDotMaxBlocks = 2048;
-constexpr int kDotUnroll = 4;
+constexpr int kDotMaxBlocks = 4096;
+constexpr int kDotUnroll = 1;
 // scratch layout: [64 B ..) kDotMaxBlocks fp32 partials (the first 64 B are unused padding)
 constexpr int64_t kDotScratchBytes = 64 + (int64_t)kDotMaxBlocks * 4;
 
@@ -90,7 +90,10 @@ __global__ __launch_bounds__(kDotThreads) void dot_kernel(const uint32_t *__rest
     }
     for (int64_t j = done + tid; j < n_words; j += nthreads) acc[0] = mac_word<KIND>(x1[j], x2[j], acc[0]);
 
-    float s = wave_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
+    float tot = acc[0];                                     // fixed order of the per-thread sums
+#pragma unroll
+    for (int u = 1; u < kDotUnroll; u++) tot += acc[u];
+    float s = wave_sum(tot);
     const int lane = lane_id(), wave = wave_id();
     if (lane == 0) wave_part[wave] = s;
     __syncthreads();

@@ -80,9 +80,12 @@ template <int MODE, int ROUND>
 static int launch_pack(const void *src, void *dst, int64_t n, hipStream_t s) {
     int64_t n16 = n / 16;
     bool al = aligned(src, 16) && aligned(dst, 16);
+    // One 16-element group per thread and as many workgroups as that takes: a grid capped at 4096 workgroups that
+    // strides over the input reached 5.2 TB/s on 134 M elements, one group per thread 6.1 TB/s (the loop in the kernel
+    // only runs more than once beyond 2^31 workgroups).
     int64_t threads_needed = n16 > 4 ? n16 : 4;
     int64_t blocks = (threads_needed + 255) / 256;
-    if (blocks > 256 * 16) blocks = 256 * 16;         // grid-stride beyond 16 workgroups per CU
+    if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
     if (blocks < 1) blocks = 1;
     if (al)
         hipLaunchKernelGGL((pack_fp8_kernel<MODE, ROUND, true>), dim3((unsigned)blocks), dim3(256), 0, s,
@@ -96,50 +99,36 @@ static int launch_pack(const void *src, void *dst, int64_t n, hipStream_t s) {
 // ---------------------------------------------------------------- fp32 -> packed fp8
 
 // The rounding chain of an fp32 producer that feeds a packed GEMV: fp32 -> fp16 (RNE) -> FP8 code
-// (RNE), four codes per word (quant4).  Thread t converts elements [16t, 16t+16) from four 128-bit
-// loads to one 128-bit store; the tail is handled one word per thread with zero padding.
+// (RNE), four codes per word (quant4).  One thread converts four elements from one 128-bit load to one
+// word: loads and stores of a wave are contiguous (16 elements per thread from four loads, each a
+// 64-byte stride apart across the lanes, ran at a third of the speed).  The last, partial word is padded with +0.
 template <int MODE, bool ALIGNED>
 __global__ __launch_bounds__(256) void quant_pack_f32_kernel(const float *__restrict__ src, uint32_t *__restrict__ dst,
-                                                            int64_t n, int64_t n16) {
-    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t g = t; g < n16; g += stride) {
-        uint32_t w[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float4_t v;
-            if constexpr (ALIGNED) v = __builtin_nontemporal_load(reinterpret_cast<const float4_t *>(src) + 4 * g + i);
-            else v = float4_t{src[16 * g + 4 * i], src[16 * g + 4 * i + 1], src[16 * g + 4 * i + 2], src[16 * g + 4 * i + 3]};
-            w[i] = quant4<MODE>(v[0], v[1], v[2], v[3]);
-        }
-        if constexpr (ALIGNED) {
-            store_nt128(reinterpret_cast<u32x4 *>(dst) + g, u32x4{w[0], w[1], w[2], w[3]});
+                                                            int64_t n) {
+    const int64_t n_words = (n + 3) / 4, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < n_words; g += stride) {
+        float4_t v;
+        if (4 * g + 3 < n) {
+            if constexpr (ALIGNED) v = __builtin_nontemporal_load(reinterpret_cast<const float4_t *>(src) + g);
+            else v = float4_t{src[4 * g], src[4 * g + 1], src[4 * g + 2], src[4 * g + 3]};
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) dst[4 * g + i] = w[i];
+            for (int i = 0; i < 4; i++) v[i] = 4 * g + i < n ? src[4 * g + i] : 0.f;
         }
-    }
-    const int64_t first = 16 * n16, tail_words = (n - first + 3) / 4;
-    if (t < tail_words) {
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) v[i] = first + 4 * t + i < n ? src[first + 4 * t + i] : 0.f;
-        dst[first / 4 + t] = quant4<MODE>(v[0], v[1], v[2], v[3]);
+        __builtin_nontemporal_store(quant4<MODE>(v[0], v[1], v[2], v[3]), dst + g);
     }
 }
 
 template <int MODE>
 static int launch_quant_pack(const void *src, void *dst, int64_t n, hipStream_t s) {
-    const int64_t n16 = n / 16;
-    const bool al = aligned(src, 16) && aligned(dst, 16);
-    int64_t blocks = ((n16 > 4 ? n16 : 4) + 255) / 256;
-    if (blocks > 256 * 16) blocks = 256 * 16;
-    if (al)
+    int64_t blocks = ((n + 3) / 4 + 255) / 256;
+    if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
+    if (aligned(src, 16))
         hipLaunchKernelGGL((quant_pack_f32_kernel<MODE, true>), dim3((unsigned)blocks), dim3(256), 0, s, (const float *)src,
-                           (uint32_t *)dst, n, n16);
+                           (uint32_t *)dst, n);
     else
         hipLaunchKernelGGL((quant_pack_f32_kernel<MODE, false>), dim3((unsigned)blocks), dim3(256), 0, s, (const float *)src,
-                           (uint32_t *)dst, n, n16);
+                           (uint32_t *)dst, n);
     return check_launch("feather_quant_pack_f32");
 }
 
@@ -185,8 +174,10 @@ __global__ __launch_bounds__(256) void unpack_fp8_kernel(const uint32_t *__restr
 
 template <int MODE, int SEM, int OUT, bool RELU>
 static int launch_unpack(const void *src, void *dst, int64_t n_words, hipStream_t s) {
-    int64_t blocks = (n_words + 255) / 256;
-    if (blocks > 256 * 32) blocks = 256 * 32;
+    // four words per thread (grid-stride): 6.0 TB/s on 134 M elements against 5.6 TB/s with a grid capped at 8192
+    // workgroups and 5.7 TB/s with one word per thread
+    int64_t blocks = (n_words + 1023) / 1024;
+    if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL((unpack_fp8_kernel<MODE, SEM, OUT, RELU>), dim3((unsigned)blocks), dim3(256), 0, s,
                        (const uint32_t *)src, dst, n_words);
@@ -248,8 +239,9 @@ __global__ __launch_bounds__(256) void copy128_kernel(const u32x4 *__restrict__ 
 // copies the first n16 16-byte units; returns how many it took (0 if the pointers are not aligned)
 static int64_t launch_copy128(const void *src, void *dst, int64_t n16, hipStream_t s) {
     if (n16 <= 0 || !aligned(src, 16) || !aligned(dst, 16)) return 0;
-    int64_t blocks = (n16 + 256 * 4 - 1) / (256 * 4);
-    if (blocks > 256 * 16) blocks = 256 * 16;
+    // one 16-byte unit per thread: 6.4 TB/s on 268 MB against 4.7 TB/s with four units per thread on a capped grid
+    int64_t blocks = (n16 + 255) / 256;
+    if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
     hipLaunchKernelGGL(copy128_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, n16);
     return n16;
 }

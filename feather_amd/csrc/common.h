@@ -164,6 +164,29 @@ __device__ __forceinline__ uint32_t enc_e4m3(uint32_t h) {
     return sign | code;
 }
 
+// Two fp16 values (one 32-bit register) -> their two E4M3fn codes in the low bytes of the two halves
+// (bits [0, 8) and [16, 24)), round to nearest even: enc_e4m3 on 16-bit lanes with packed instructions, both
+// paths computed and merged bit-wise instead of a branch per element (random data takes both branches in every
+// wave: the scalar encoder made the E4M3 pack kernel VALU bound, 5.0 TB/s against 6.1 TB/s for E5M2).
+//   |x| >= 2^-6 (bits >= 0x2400): rebias, add 0x3F + lsb, shift: a carry moves into the exponent; capped at 0x7F
+//   |x| <  2^-6: the code is round-to-nearest-even(|x| * 2^9), read from the low bits of |x| * 512 + 1024 in
+//                fp16 arithmetic (the product is exact, and the ulp at 1024 is 1)
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t enc_e4m3_pair(uint32_t hh) {
+    const uint32_t a32 = hh & 0x7FFF7FFFu;
+    const u16x2_t a = __builtin_bit_cast(u16x2_t, a32);
+    u16x2_t t = a - (uint16_t)0x2000;
+    t = t + (uint16_t)0x3F + ((t >> (uint16_t)7) & (uint16_t)1);
+    const u16x2_t norm = __builtin_elementwise_min((u16x2_t)(t >> (uint16_t)7), (u16x2_t)(uint16_t)0x7F);
+    const half2_t scaled = __builtin_elementwise_fma(as_half2(a32), (half2_t)(_Float16)512.0f, (half2_t)(_Float16)1024.0f);
+    const uint32_t sub = as_u32(scaled) & 0x000F000Fu;
+    // all-ones halves where |x| >= 2^-6: a + 0x5C00 has bit 15 set exactly then (a <= 0x7FFF: no wrap)
+    const u16x2_t big = (u16x2_t)((a + (uint16_t)0x5C00) >> (uint16_t)15) * (uint16_t)0xFFFF;
+    const uint32_t m = __builtin_bit_cast(uint32_t, big);
+    const uint32_t mag = (__builtin_bit_cast(uint32_t, norm) & m) | (sub & ~m);
+    return mag | ((hh >> 8) & 0x00800080u);
+}
+
 template <int MODE, int ROUND>
 __device__ __forceinline__ uint32_t enc(uint32_t h) {
     if constexpr (ROUND == FEATHER_ROUND_TRUNC) return (h >> 8) & 0xFFu;
@@ -184,8 +207,8 @@ __device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d) {
     uint32_t h2 = __builtin_bit_cast(uint16_t, (_Float16)c), h3 = __builtin_bit_cast(uint16_t, (_Float16)d);
     if constexpr (MODE == FEATHER_E5M2)
         return enc_e5m2(h0) | (enc_e5m2(h1) << 8) | (enc_e5m2(h2) << 16) | (enc_e5m2(h3) << 24);
-    else
-        return enc_e4m3(h0) | (enc_e4m3(h1) << 8) | (enc_e4m3(h2) << 16) | (enc_e4m3(h3) << 24);
+    else   // two elements per instruction; the codes come back in bytes 0 and 2 of each pair
+        return perm(enc_e4m3_pair(h2 | (h3 << 16)), enc_e4m3_pair(h0 | (h1 << 16)), 0x06040200u);
 }
 
 // the four fp16 values that a packed word decodes to (kernel decode), as two fp16 pairs

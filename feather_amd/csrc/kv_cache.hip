@@ -40,6 +40,7 @@ __global__ __launch_bounds__(256) void paged_cache_write_kernel(
         if constexpr (F16) {
             const u32x4 a = reinterpret_cast<const u32x4 *>(sp)[2 * src], b = reinterpret_cast<const u32x4 *>(sp)[2 * src + 1];
             auto enc4 = [](uint32_t p01, uint32_t p23) {            // two words of fp16 pairs -> one packed word
+                if constexpr (MODE == FEATHER_E4M3) return perm(enc_e4m3_pair(p23), enc_e4m3_pair(p01), 0x06040200u);
                 return enc<MODE, FEATHER_ROUND_RNE>(p01 & 0xFFFFu) | (enc<MODE, FEATHER_ROUND_RNE>(p01 >> 16) << 8) |
                        (enc<MODE, FEATHER_ROUND_RNE>(p23 & 0xFFFFu) << 16) | (enc<MODE, FEATHER_ROUND_RNE>(p23 >> 16) << 24);
             };

@@ -52,8 +52,12 @@ __global__ __launch_bounds__(256) void pack_fp8_kernel(const uint16_t *__restric
         }
         uint32_t w[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            w[i] = enc_pair<MODE, ROUND>(in[2 * i]) | (enc_pair<MODE, ROUND>(in[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; i++) {
+            if constexpr (MODE == FEATHER_E4M3 && ROUND == FEATHER_ROUND_RNE)   // codes in bytes 0 and 2 of each register
+                w[i] = perm(enc_e4m3_pair(in[2 * i + 1]), enc_e4m3_pair(in[2 * i]), 0x06040200u);
+            else
+                w[i] = enc_pair<MODE, ROUND>(in[2 * i]) | (enc_pair<MODE, ROUND>(in[2 * i + 1]) << 16);
+        }
         if constexpr (ALIGNED) {
             store_nt128(reinterpret_cast<u32x4 *>(dst) + g, u32x4{w[0], w[1], w[2], w[3]});
         } else {

@@ -157,9 +157,20 @@ __global__ __launch_bounds__(256) void unpack_fp8_kernel(const uint32_t *__restr
     int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t j = t; j < n_words; j += stride) {
         uint32_t w = __builtin_nontemporal_load(src + j);
-        uint32_t p01, p23;
-        dec_word_sem<MODE, SEM>(w, p01, p23);
-        half2_t a = as_half2(p01), b = as_half2(p23);
+        half2_t a, b;
+        if constexpr (MODE == FEATHER_E4M3 && SEM == FEATHER_SEM_IEEE) {
+            // the matrix core's FP8 format is the OCP E4M3fn of the CPU API's decode (subnormals m * 2^-9, 0x7F / 0xFF
+            // NaN): the hardware conversion does the whole word in two instructions; every value is exact in fp16
+            typedef float float2_t __attribute__((ext_vector_type(2)));
+            const float2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+            a = half2_t{(_Float16)lo[0], (_Float16)lo[1]};
+            b = half2_t{(_Float16)hi[0], (_Float16)hi[1]};
+        } else {
+            uint32_t p01, p23;
+            dec_word_sem<MODE, SEM>(w, p01, p23);
+            a = as_half2(p01);
+            b = as_half2(p23);
+        }
         if constexpr (RELU) {
             // max(0, x) as in tl.maximum(0.0, x): a negative or NaN-free compare
             a.x = a.x > (_Float16)0 ? a.x : (_Float16)0;

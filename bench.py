@@ -391,7 +391,7 @@ def main() -> int:
             extra[key + "_tokens_per_s"] = round(batch / us * 1e6, 0)
             extra[key + "_GBps"] = round(step_bytes / us / 1e3, 1)
             rl[key] = roofline_record(ttab, key, "feather_decode_step (all kernels of one step)", step_bytes, us,
-                                      launches_per_call=10 * cfg.n_layers + 3)
+                                      launches_per_call=8 * cfg.n_layers + 3)
             del dec, logits, btd
             torch.cuda.empty_cache()
 

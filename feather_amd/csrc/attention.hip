@@ -35,10 +35,13 @@
 // rounded to fp16 before P.V, fp32 output.  One difference inside the stated
 // tolerance: the denominator sums the fp16-rounded P (the values that multiply
 // V) where the reference sums P before rounding.
+#include <cstdlib>
 #include <type_traits>
 #include "common.h"
 
 namespace feather {
+
+typedef float float2v_t __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float4_t mfma16(half8_t a, half8_t b, float4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -518,6 +521,265 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     }
 }
 
+// ---- d = 64, E5M2: the FP8-rate kernel -------------------------------------------------------------
+// Same work split, staging and numerics as flash_attn_kernel<64, E5M2, ...> (a wave owns 64 queries,
+// 64-key tiles, K staged as raw bytes, V^T as fp16), on the 32x32 matrix instructions:
+//     S^T[32 keys, 32 q]  = v_mfma_f32_32x32x64_f8f6f4 (both operands BF8 = E5M2): the whole head dim in
+//                           one instruction at the FP8 rate, 4 per tile where the 16x16x32 form needs 32;
+//     O^T[32 dd, 32 q]   += v_mfma_f32_32x32x16_f16, 16 per tile.
+// What it buys is vector-ALU issue time, which bounds this head dim: an MFMA holds the SIMD's vector
+// issue for as long as its operands take to read (measured: 8 cycles for a 16x16x32 fp16 MFMA, 4 for
+// the bf8 one, about the same 8 for a 32x32x16 that does twice the work), so 20 large MFMAs per tile
+// block it for ~170 cycles where 72 small ones block it for ~450; a query is shared by two lanes
+// instead of four (one cross-lane step per maximum instead of two), and the row sums are two-term dot
+// products on the fp16 pairs of P (v_dot2_f32_f16, 32 per tile) instead of a constant-ones MFMA whose
+// 32x32 form would cost 32 accumulator registers.
+// Layouts (lane l, n = l % 32, h = l / 32): an MFMA operand row is [n]; operand bytes / halves are the
+// k-slots 32 h .. 32 h + 31 (f8f6f4) or 8 h .. 8 h + 7 (f16); accumulator register r of a 32x32 block is
+// row 8 (r / 4) + 4 h + r % 4, column n.  So a lane holds, for query n, the scores of keys
+// 8 g + 4 h + {0..3} (g = 0..3) of each 32-key block, and registers 8 s .. 8 s + 7 are exactly the eight
+// k-slots the second MFMA wants from this lane for the 16-key step s if V^T stores the keys of every
+// group of 16 in the order 0 1 2 3 8 9 10 11 | 4 5 6 7 12 13 14 15.  (Both operands of the score MFMA take
+// the same bytes of a row, so the order of the k-slots inside the instruction does not matter.)
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef int int8v_t __attribute__((ext_vector_type(8)));
+
+template <bool VC, int WAVES, int OCC>
+__global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
+    const uint32_t *__restrict__ q, const uint32_t *__restrict__ k, const uint32_t *__restrict__ v,
+    float *__restrict__ out, int L, int n_heads, int kv_group, int tiles_per_head, float scale_log2e,
+    int keys_scored, int mask_tail, const int32_t *__restrict__ cu_seqlens, int tiles_per_seq, int total_rows,
+    int causal) {
+    constexpr int D = 64, DW = 16, BN = 64;
+    constexpr int KP = D + 16;             // K row pitch in LDS, bytes
+    constexpr int VS = BN;                 // fp16 per V^T row
+    constexpr int kThreads = 64 * WAVES, QT = 64 * WAVES;
+    constexpr int UNITS = BN * D / 16;     // 16-code units of a K (or V) tile: 256
+    static_assert(UNITS <= kThreads && UNITS % 64 == 0, "the first UNITS threads stage a tile");
+    constexpr int kBufBytes = BN * KP + D * VS * 2;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // V^T swizzle: 16-byte chunk c of row r lives at chunk c ^ swz(r).  The 16 lanes of a fragment read take
+    // the same chunk of 16 consecutive rows (distinct bank groups for rows of equal parity need distinct
+    // swz over r / 2 % 8); the writers of a wave take rows 4 apart (bits 2..5 of the row vary)
+    auto swz = [](int row) { return ((row >> 1) & 7) ^ ((row >> 4) & 1); };
+
+    int bid = blockIdx.x;
+    const int total = gridDim.x;
+    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;   // an XCD works through contiguous (head, tile) pairs
+    const int head = bid / tiles_per_head;
+    int tile = bid % tiles_per_head;
+    const int kv_head = head / kv_group;
+    int64_t q_row0 = (int64_t)head * L, kv_row0 = (int64_t)kv_head * L;
+    if constexpr (VC) {
+        const int seq = tile / tiles_per_seq;
+        tile = tile % tiles_per_seq;
+        if (causal) tile = tiles_per_seq - 1 - tile;          // the tiles with the longest key loops start first
+        const int r0 = cu_seqlens[seq];
+        L = cu_seqlens[seq + 1] - r0;
+        if (tile * QT >= L) return;
+        q_row0 = (int64_t)head * total_rows + r0;
+        kv_row0 = (int64_t)kv_head * total_rows + r0;
+        mask_tail = 1;
+        const int last_key = causal ? min(L, (tile + 1) * QT) : L;
+        keys_scored = (last_key + BN - 1) / BN * BN;
+    }
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = wave_id();
+    const int n = lane & 31, h = lane >> 5;
+    const int q0 = tile * QT + wave * 64;
+    const uint32_t *qh = q + q_row0 * DW;
+    const uint32_t *kh = k + kv_row0 * DW;
+    const uint32_t *vh = v + kv_row0 * DW;
+
+    // ---- Q operands: 32 bytes of the lane's query row per 32-query block
+    int8v_t qf[2];
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+        const int row = q0 + 32 * b + n;
+        u32x4 w0 = u32x4{0, 0, 0, 0}, w1 = u32x4{0, 0, 0, 0};
+        if (row < L) {
+            const u32x4 *src = reinterpret_cast<const u32x4 *>(qh + (int64_t)row * DW + 8 * h);
+            w0 = src[0];
+            w1 = src[1];
+        }
+        qf[b] = int8v_t{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+    }
+
+    constexpr float kLazy = 8.f;
+    const float lazy_raw = kLazy / scale_log2e;   // the same margin in raw-score units
+    float16_t o[2][2];      // [query block][32-dim block]
+    float m_run[2], l_run[2];   // running maximum of the query; the lane's share of its row sum
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+        m_run[b] = -INFINITY;
+        l_run[b] = 0.f;
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[b][d][r] = 0.f;
+    }
+
+    // ---- register staging of the next packed K / V tile (the first UNITS threads)
+    u32x4 kreg;
+    uint32_t vreg[4];
+    auto prefetch = [&](int key0) {
+        if (UNITS < kThreads && tid >= UNITS) return;
+        const int row0 = __builtin_amdgcn_readfirstlane(key0);
+        const char *kt = reinterpret_cast<const char *>(kh + (int64_t)row0 * DW);
+        const char *vt = reinterpret_cast<const char *>(vh + (int64_t)row0 * DW);
+        int t = tid;
+        asm volatile("" : "+v"(t));   // keeps base + offset from being hoisted out of the key loop as 64-bit pairs
+        const int krel = t / 4, c16 = t % 4;
+        kreg = u32x4{0, 0, 0, 0};
+        if (key0 + krel < L) kreg = *reinterpret_cast<const u32x4 *>(kt + (uint32_t)(krel * D + 16 * c16));
+        const int ddw = t % DW, kg = t / DW;
+        const uint32_t voff = (uint32_t)(4 * kg * D + 4 * ddw);
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            vreg[r] = key0 + 4 * kg + r < L ? *reinterpret_cast<const uint32_t *>(vt + voff + (uint32_t)(r * D)) : 0u;
+    };
+    auto stage = [&](int buf) {
+        if (UNITS < kThreads && tid >= UNITS) return;
+        unsigned char *k_lds = smem + buf * kBufBytes;
+        _Float16 *vt_lds = reinterpret_cast<_Float16 *>(k_lds + BN * KP);
+        const int key = tid / 4, c16 = tid % 4;
+        *reinterpret_cast<u32x4 *>(k_lds + key * KP + 16 * c16) = kreg;
+        // V: 4 keys x 4 dims -> V^T[dd][slot]; keys 4 kg .. 4 kg + 3 are quarter q4 = kg % 4 of their group of
+        // 16 and go to slots 8 (q4 & 1) + 4 (q4 >> 1) .. + 3 of it
+        const int ddw = tid % DW, kg = tid / DW;
+        const int q4 = kg & 3, pos = 16 * (kg >> 2) + 8 * (q4 & 1) + 4 * (q4 >> 1);
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            // halfs (key r, key r + 1) of dim 4 ddw + c: byte c of each word, placed as the high byte
+            const uint32_t sel = 0x000c000cu | ((uint32_t)c << 8) | ((uint32_t)(4 + c) << 24);
+            const uint32_t lo2 = perm(vreg[1], vreg[0], sel), hi2 = perm(vreg[3], vreg[2], sel);
+            const int row = 4 * ddw + c;
+            *reinterpret_cast<u32x2 *>(vt_lds + row * VS + (((pos >> 3) ^ swz(row)) << 3) + (pos & 4)) = u32x2{lo2, hi2};
+        }
+    };
+
+    prefetch(0);
+    stage(0);
+    if (BN < keys_scored) prefetch(BN);
+    __syncthreads();
+    int cur = 0;
+    for (int key0 = 0; key0 < keys_scored; key0 += BN, cur ^= 1) {
+        if (key0 + BN < keys_scored) {
+            stage(cur ^ 1);
+            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
+        }
+        const unsigned char *k_lds = smem + cur * kBufBytes;
+        const _Float16 *vt_lds = reinterpret_cast<const _Float16 *>(k_lds + BN * KP);
+        const bool ragged = mask_tail && key0 + BN > L;   // only the last tile can hold masked keys
+        bool diag = false, skip = false;
+        if constexpr (VC) {
+            diag = causal && key0 + BN - 1 > q0;          // some key of the tile lies past the wave's first query
+            skip = causal && key0 > q0 + 63;              // every key lies past the wave's last query
+        }
+        if (!skip) {
+            // ---- S^T = K Q^T, raw scores: [query block][key block]
+            int8v_t kf[2];
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const u32x4 *src = reinterpret_cast<const u32x4 *>(k_lds + (32 * c + n) * KP + 32 * h);
+                const u32x4 w0 = src[0], w1 = src[1];
+                kf[c] = int8v_t{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+            }
+            half8_t vf[4][2];   // [16-key step][32-dim block]
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int d = 0; d < 2; d++) {
+                    const int row = 32 * d + n;
+                    vf[g][d] = *reinterpret_cast<const half8_t *>(vt_lds + row * VS + (((2 * g + h) ^ swz(row)) << 3));
+                }
+            float16_t sc[2][2];
+            const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+#pragma unroll
+                for (int c = 0; c < 2; c++)   // cbsz = blgp = 1: both operands are BF8 (E5M2); no block scales
+                    sc[b][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[c], qf[b], zero16, 1, 1, 0, 0, 0, 0);
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                // ---- online softmax of one 32-query block; p = 2^(s * c - m * c) on the raw-score maximum
+                if (ragged || diag) {
+                    int last = diag ? min(L - 1, q0 + 32 * b + n) : L - 1;   // last visible key
+                    asm volatile("" : "+v"(last));   // keeps the 32 compares inside this rarely taken branch
+                    const int rel = last - key0 - 4 * h;   // key 32 c + 8 (r / 4) + 4 h + r % 4 is hidden if 32 c + 8 (r / 4) + r % 4 > rel
+#pragma unroll
+                    for (int c = 0; c < 2; c++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++)
+                            if (32 * c + 8 * (r >> 2) + (r & 3) > rel) sc[b][c][r] = -INFINITY;
+                }
+                float mx = max3_raw(sc[b][0][0], sc[b][0][1], sc[b][0][2]);
+                mx = max_raw(mx, sc[b][0][3]);
+#pragma unroll
+                for (int i = 2; i < 16; i++) mx = max3_raw(mx, sc[b][i >> 3][(2 * i) & 15], sc[b][i >> 3][(2 * i + 1) & 15]);
+                mx = max_xor32(mx);   // the two lanes that share the query
+                // The reference point of the exponentials is a running maximum that is only raised when some
+                // query of the block exceeds it by more than kLazy binary orders of magnitude: P then lies in
+                // (0, 2^kLazy] instead of (0, 1], which fp16 holds with the same relative precision, the
+                // quotient O / l does not depend on the reference point, and the rescaling of the block's
+                // 34 accumulator registers runs for a few tiles per sequence instead of for most of them
+                // (a block of 32 queries of random data sees a new maximum in ~60 % of 128 tiles).
+                if (__builtin_amdgcn_ballot_w64(mx > m_run[b] + lazy_raw) != 0) {
+                    const float m_old = m_run[b];
+                    const float m_new = max_raw(m_old, mx);
+                    const float alpha = __builtin_amdgcn_exp2f((m_old - m_new) * scale_log2e);
+                    m_run[b] = m_new;
+                    l_run[b] *= alpha;
+#pragma unroll
+                    for (int d = 0; d < 2; d++) o[b][d] *= alpha;
+                }
+                const float mc = m_run[b] * scale_log2e;
+                half8_t pb[4];
+                float lsum = 0.f;
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    uint32_t pw[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {   // P rounded to fp16 (nearest even), as P.to(fp16)
+                        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[b][g >> 1][8 * (g & 1) + 2 * i], scale_log2e, -mc));
+                        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[b][g >> 1][8 * (g & 1) + 2 * i + 1], scale_log2e, -mc));
+                        pw[i] = as_u32(__builtin_convertvector(float2v_t{e0, e1}, half2_t));
+                        lsum = dot2(pw[i], 0x3c003c00u, lsum);   // the row sum takes the rounded values that multiply V
+                    }
+                    pb[g] = __builtin_bit_cast(half8_t, u32x4{pw[0], pw[1], pw[2], pw[3]});
+                }
+                l_run[b] += lsum;
+                // ---- O^T += V^T P^T
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+#pragma unroll
+                    for (int d = 0; d < 2; d++)
+                        o[b][d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[g][d], pb[g], o[b][d], 0, 0, 0);
+            }
+        }
+        __syncthreads();  // tile i+1 is visible; every wave is done reading tile i
+    }
+
+    // ---- epilogue: the two lanes of a query add their shares of the row sum; normalise, store [q][dd]
+    float *oh = out + q_row0 * D;
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+        const float other = as_float((uint32_t)__builtin_amdgcn_ds_bpermute(4 * (lane ^ 32), (int)as_u32(l_run[b])));
+        const float l = l_run[b] + other;
+        const int row = q0 + 32 * b + n;
+        if (row < L) {
+#pragma unroll
+            for (int d = 0; d < 2; d++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const float4_t x = {o[b][d][4 * g], o[b][d][4 * g + 1], o[b][d][4 * g + 2], o[b][d][4 * g + 3]};
+                    *reinterpret_cast<float4_t *>(oh + (int64_t)row * D + 32 * d + 8 * g + 4 * h) = x / l;
+                }
+        }
+    }
+}
+
 // Fixed-length heads (cu_seqlens == nullptr; L rows per head) or packed variable-length sequences
 // (cu_seqlens given: n_seq sequences of at most max_seqlen rows inside total_rows rows per head).
 struct AttnArgs {
@@ -558,6 +820,27 @@ static int launch_attn(const AttnArgs &a, hipStream_t s) {
     return check_launch("feather_flash_attn_fp8");
 }
 
+template <bool VC, int WAVES, int OCC>
+static int launch_attn64_bf8(const AttnArgs &a, hipStream_t s) {
+    constexpr int QT = 64 * WAVES, BN = 64, D = 64;
+    constexpr size_t lds = (size_t)(BN * (D + 16) + D * BN * 2) * 2;   // two (K bytes, V^T fp16) buffers
+    const int64_t L = VC ? a.max_seqlen : a.L;
+    const int tiles_per_seq = (int)((L + QT - 1) / QT);
+    const int64_t tiles = VC ? tiles_per_seq * a.n_seq : tiles_per_seq;
+    const int64_t blocks = tiles * a.n_heads;
+    FEATHER_CHECK(blocks < (1ll << 31), FEATHER_ESHAPE, "feather_flash_attn_fp8: grid too large");
+    if (blocks == 0) return FEATHER_OK;
+    // both tail modes score whole 64-key tiles here (the reference scores zero rows past L, the mask hides them)
+    const int64_t keys_scored = (L + BN - 1) / BN * BN;
+    const float log2e = 1.4426950408889634f;
+    hipLaunchKernelGGL((flash_attn64_bf8_kernel<VC, WAVES, OCC>), dim3((unsigned)blocks), dim3(64 * WAVES), lds, s,
+                       (const uint32_t *)a.q, (const uint32_t *)a.k, (const uint32_t *)a.v, (float *)a.out, (int)L,
+                       (int)a.n_heads, (int)a.kv_group, (int)tiles, a.scale * log2e, (int)keys_scored,
+                       a.tail == FEATHER_TAIL_MASK ? 1 : 0, (const int32_t *)a.cu_seqlens, tiles_per_seq,
+                       (int)a.total_rows, a.causal);
+    return check_launch("feather_flash_attn_fp8");
+}
+
 // Workgroup shapes.  A wave of the d = 64 kernel owns 64 queries.  Staging a K/V tile into LDS is
 // shared by the workgroup's waves, and from d = 128 on it is a large share of the vector work, so
 // eight waves (twice the queries per staged tile, two waves per SIMD from one workgroup to overlap
@@ -576,6 +859,10 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
         case 64:   // all four query blocks of a wave share every K fragment
             // eight waves halve the staging work per query (-2 % time); a causal tile of 512 queries
             // would idle its early waves through too many masked key tiles
+            if constexpr (MODE == FEATHER_E5M2) if (!getenv("FEATHER_EXP_ATTN64_OLD")) {   // the FP8-rate kernel, same two workgroup shapes
+                if (!a.causal && fills_chip(512)) return launch_attn64_bf8<VC, 8, 1>(a, s);
+                return launch_attn64_bf8<VC, 4, 2>(a, s);
+            }
             if (!a.causal && fills_chip(512)) return launch_attn<64, MODE, 4, 4, 64, 1, VC, 8>(a, s);
             return launch_attn<64, MODE, 4, 4, 64, 2, VC>(a, s);
         case 128:

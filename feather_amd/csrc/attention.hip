@@ -35,7 +35,6 @@
 // rounded to fp16 before P.V, fp32 output.  One difference inside the stated
 // tolerance: the denominator sums the fp16-rounded P (the values that multiply
 // V) where the reference sums P before rounding.
-#include <cstdlib>
 #include <type_traits>
 #include "common.h"
 
@@ -174,6 +173,8 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
 #pragma unroll
         for (int d = 0; d <= DB; d++) o[b][d] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
+    constexpr float kLazy = 8.f;
+    const float lazy_raw = kLazy / scale_log2e;   // the same margin in raw-score units
     const _Float16 one_or_zero = (j & 3) == 0 ? (_Float16)1 : (_Float16)0;
     const half8_t ones = {one_or_zero, one_or_zero, one_or_zero, one_or_zero,
                           one_or_zero, one_or_zero, one_or_zero, one_or_zero};
@@ -308,8 +309,14 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                 mx = max3_raw(mx, sb[c][2], sb[c][3]);
             }
             mx = max_xor32(max_xor16(mx));   // over the four lanes that share the query
+            // The reference point of the exponentials is only raised when some query of the block exceeds it by
+            // more than kLazy binary orders of magnitude (P then lies in (0, 2^kLazy], which fp16 holds with the
+            // same relative precision; O / l does not depend on the reference point): the rescaling of the
+            // block's 4 (DB + 1) accumulator registers, more than its whole softmax from d = 256 on, runs for
+            // a few tiles per sequence instead of for a third of them.
             const float m_old = m_run[qb];
-            const float m_new = max_raw(m_old, mx);
+            const bool raise = __builtin_amdgcn_ballot_w64(mx > m_old + lazy_raw) != 0;
+            const float m_new = raise ? max_raw(m_old, mx) : m_old;
             const float mc = m_new * scale_log2e;
             if constexpr (K16) {
                 half4_t p4;
@@ -331,64 +338,13 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                     pb[t] = p8;
                 }
             }
-            // rescale only when some query of this block saw a new maximum (wave-uniform test)
-            if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
+            if (raise) {   // wave-uniform
                 const float alpha = __builtin_amdgcn_exp2f((m_old - m_new) * scale_log2e);
                 m_run[qb] = m_new;
 #pragma unroll
                 for (int d = 0; d <= DB; d++) o[qb][d] *= alpha;
             }
         };
-        // PVB: with several query blocks per wave, one-byte (bf8) K fragments and K / V^T tiles small
-        // enough to sit in registers (d = 64: 8 + 8 fragments), the blocks go through score -> softmax ->
-        // P.V one after the other with the scores one block ahead: the MFMAs of block b's P.V and of
-        // block b + 2's scores run on the matrix core while the vector ALU works through block b + 1's
-        // exponentials (d = 64, L = 8192: 1189 -> 1147 us).  The fp16 score path has no registers left
-        // for resident K fragments (spills) and re-reading them from LDS per block costs more than the
-        // overlap gains (1250 -> 1262 / 1275 us), so there, and for the wider heads, all blocks share
-        // each K / V^T fragment as it is read from LDS.  (s_setprio 1 around the MFMA groups, or around
-        // the softmax instead, to steer which of a SIMD's two waves issues: 1163 / 1182 us against 1143;
-        // and a run that skipped every other tile barrier, wrong results, was only 1.2 % faster.)
-        constexpr bool PVB = KSPLIT == 1 && BF8 && QB > 1 && DB * KB32 <= 8 && KB16 * STEPS <= 8;
-        if constexpr (PVB) {
-            long kres[KB16][STEPS];
-            half8_t vres[KB32][DB];
-#pragma unroll
-            for (int c = 0; c < KB16; c++)
-#pragma unroll
-                for (int st = 0; st < STEPS; st++)
-                    kres[c][st] = *reinterpret_cast<const long *>(reinterpret_cast<const unsigned char *>(k_lds) +
-                                                                  (16 * c + j) * (2 * KS) + 32 * st + 8 * kb);
-#pragma unroll
-            for (int t = 0; t < KB32; t++)
-#pragma unroll
-                for (int d = 0; d < DB; d++)
-                    vres[t][d] = *reinterpret_cast<const half8_t *>(vt_lds + (16 * d + j) * VS +
-                                                                    (((4 * t + kb) ^ swz(16 * d + j)) << 3));
-            float4_t s2[2][KB16];
-            auto score = [&](int qb, float4_t (&sb)[KB16]) {
-#pragma unroll
-                for (int c = 0; c < KB16; c++)
-#pragma unroll
-                    for (int st = 0; st < STEPS; st++) {
-                        const float4_t acc0 = st == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : sb[c];
-                        sb[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(kres[c][st], qf8[qb][st], acc0, 0, 0, 0);
-                    }
-            };
-            score(0, s2[0]);
-#pragma unroll
-            for (int b = 0; b < QB; b++) {
-                if (b + 1 < QB) score(b + 1, s2[(b + 1) & 1]);
-                half8_t pb[KB32];
-                softmax_block(b, s2[b & 1], pb);
-#pragma unroll
-                for (int t = 0; t < KB32; t++) {
-#pragma unroll
-                    for (int d = 0; d < DB; d++) o[b][d] = mfma16(vres[t][d], pb[t], o[b][d]);
-                    o[b][DB] = mfma16(ones, pb[t], o[b][DB]);
-                }
-            }
-        } else {
         pfrag_t pf[QB][GKB32];
         const int kc0 = kgroup * GKB16;   // first 16-key block of this key group inside the tile
         // query blocks are scored SB at a time: the K fragments are re-used across the SB
@@ -449,7 +405,6 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
             for (int b = 0; b < QB; b++) o[b][DB] = mfma16(ones, pf[b][t], o[b][DB]);
         }
         }
-        }   // !PVB
         }   // !skip
         if (math_first && key0 + BN < keys_scored) {
             stage(cur ^ 1);
@@ -620,42 +575,61 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
             for (int r = 0; r < 16; r++) o[b][d][r] = 0.f;
     }
 
-    // ---- register staging of the next packed K / V tile (the first UNITS threads)
+    // ---- register staging of the next packed K / V tile: 256 threads carry V (4 keys x 4 dims each), 256 threads
+    // K (16 bytes of one key each): the same threads in a four-wave workgroup, waves 0-3 and 4-7 in an
+    // eight-wave one (all of them then have staging work to fill the wait for the tile's first LDS reads)
+    constexpr bool kSplitStaging = kThreads >= 2 * UNITS;
+    const bool stages_v = tid < UNITS, stages_k = kSplitStaging ? (tid >= UNITS && tid < 2 * UNITS) : tid < UNITS;
+    const int kt_id = kSplitStaging ? tid - UNITS : tid;   // index of the thread among the K stagers
     u32x4 kreg;
     uint32_t vreg[4];
     auto prefetch = [&](int key0) {
-        if (UNITS < kThreads && tid >= UNITS) return;
         const int row0 = __builtin_amdgcn_readfirstlane(key0);
         const char *kt = reinterpret_cast<const char *>(kh + (int64_t)row0 * DW);
         const char *vt = reinterpret_cast<const char *>(vh + (int64_t)row0 * DW);
-        int t = tid;
-        asm volatile("" : "+v"(t));   // keeps base + offset from being hoisted out of the key loop as 64-bit pairs
-        const int krel = t / 4, c16 = t % 4;
-        kreg = u32x4{0, 0, 0, 0};
-        if (key0 + krel < L) kreg = *reinterpret_cast<const u32x4 *>(kt + (uint32_t)(krel * D + 16 * c16));
-        const int ddw = t % DW, kg = t / DW;
-        const uint32_t voff = (uint32_t)(4 * kg * D + 4 * ddw);
+        const bool whole = key0 + BN <= L;   // wave-uniform: only the last tile needs per-row guards
+        if (stages_k) {
+            int t = kt_id;
+            asm volatile("" : "+v"(t));   // keeps base + offset from being hoisted out of the key loop as 64-bit pairs
+            const int krel = t / 4, c16 = t % 4;
+            kreg = u32x4{0, 0, 0, 0};
+            if (whole || key0 + krel < L) kreg = *reinterpret_cast<const u32x4 *>(kt + (uint32_t)(krel * D + 16 * c16));
+        }
+        if (stages_v) {
+            int t = tid;
+            asm volatile("" : "+v"(t));
+            const int ddw = t % DW, kg = t / DW;
+            const uint32_t voff = (uint32_t)(4 * kg * D + 4 * ddw);
+            if (whole) {
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-            vreg[r] = key0 + 4 * kg + r < L ? *reinterpret_cast<const uint32_t *>(vt + voff + (uint32_t)(r * D)) : 0u;
+                for (int r = 0; r < 4; r++) vreg[r] = *reinterpret_cast<const uint32_t *>(vt + voff + (uint32_t)(r * D));
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    vreg[r] = key0 + 4 * kg + r < L ? *reinterpret_cast<const uint32_t *>(vt + voff + (uint32_t)(r * D)) : 0u;
+            }
+        }
     };
     auto stage = [&](int buf) {
-        if (UNITS < kThreads && tid >= UNITS) return;
         unsigned char *k_lds = smem + buf * kBufBytes;
         _Float16 *vt_lds = reinterpret_cast<_Float16 *>(k_lds + BN * KP);
-        const int key = tid / 4, c16 = tid % 4;
-        *reinterpret_cast<u32x4 *>(k_lds + key * KP + 16 * c16) = kreg;
-        // V: 4 keys x 4 dims -> V^T[dd][slot]; keys 4 kg .. 4 kg + 3 are quarter q4 = kg % 4 of their group of
-        // 16 and go to slots 8 (q4 & 1) + 4 (q4 >> 1) .. + 3 of it
-        const int ddw = tid % DW, kg = tid / DW;
-        const int q4 = kg & 3, pos = 16 * (kg >> 2) + 8 * (q4 & 1) + 4 * (q4 >> 1);
+        if (stages_k) {
+            const int key = kt_id / 4, c16 = kt_id % 4;
+            *reinterpret_cast<u32x4 *>(k_lds + key * KP + 16 * c16) = kreg;
+        }
+        if (stages_v) {
+            // V: 4 keys x 4 dims -> V^T[dd][slot]; keys 4 kg .. 4 kg + 3 are quarter q4 = kg % 4 of their group of
+            // 16 and go to slots 8 (q4 & 1) + 4 (q4 >> 1) .. + 3 of it
+            const int ddw = tid % DW, kg = tid / DW;
+            const int q4 = kg & 3, pos = 16 * (kg >> 2) + 8 * (q4 & 1) + 4 * (q4 >> 1);
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            // halfs (key r, key r + 1) of dim 4 ddw + c: byte c of each word, placed as the high byte
-            const uint32_t sel = 0x000c000cu | ((uint32_t)c << 8) | ((uint32_t)(4 + c) << 24);
-            const uint32_t lo2 = perm(vreg[1], vreg[0], sel), hi2 = perm(vreg[3], vreg[2], sel);
-            const int row = 4 * ddw + c;
-            *reinterpret_cast<u32x2 *>(vt_lds + row * VS + (((pos >> 3) ^ swz(row)) << 3) + (pos & 4)) = u32x2{lo2, hi2};
+            for (int c = 0; c < 4; c++) {
+                // halfs (key r, key r + 1) of dim 4 ddw + c: byte c of each word, placed as the high byte
+                const uint32_t sel = 0x000c000cu | ((uint32_t)c << 8) | ((uint32_t)(4 + c) << 24);
+                const uint32_t lo2 = perm(vreg[1], vreg[0], sel), hi2 = perm(vreg[3], vreg[2], sel);
+                const int row = 4 * ddw + c;
+                *reinterpret_cast<u32x2 *>(vt_lds + row * VS + (((pos >> 3) ^ swz(row)) << 3) + (pos & 4)) = u32x2{lo2, hi2};
+            }
         }
     };
 
@@ -663,12 +637,10 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
     stage(0);
     if (BN < keys_scored) prefetch(BN);
     __syncthreads();
-    int cur = 0;
-    for (int key0 = 0; key0 < keys_scored; key0 += BN, cur ^= 1) {
-        if (key0 + BN < keys_scored) {
-            stage(cur ^ 1);
-            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
-        }
+    // One key tile; the buffer index is a compile-time constant (the loop below is unrolled by two), so every
+    // LDS address is a loop-invariant per-lane register plus an immediate offset instead of vector adds per tile.
+    auto tile_body = [&](const int key0, auto cur_c) {
+        constexpr int cur = decltype(cur_c)::value;
         const unsigned char *k_lds = smem + cur * kBufBytes;
         const _Float16 *vt_lds = reinterpret_cast<const _Float16 *>(k_lds + BN * KP);
         const bool ragged = mask_tail && key0 + BN > L;   // only the last tile can hold masked keys
@@ -677,7 +649,10 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
             diag = causal && key0 + BN - 1 > q0;          // some key of the tile lies past the wave's first query
             skip = causal && key0 > q0 + 63;              // every key lies past the wave's last query
         }
-        if (!skip) {
+        if (skip) {   // nothing to score for this wave; the other waves still need the next tile
+            if (key0 + BN < keys_scored) stage(cur ^ 1);
+            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
+        } else {
             // ---- S^T = K Q^T, raw scores: [query block][key block]
             int8v_t kf[2];
 #pragma unroll
@@ -694,6 +669,8 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
                     const int row = 32 * d + n;
                     vf[g][d] = *reinterpret_cast<const half8_t *>(vt_lds + row * VS + (((2 * g + h) ^ swz(row)) << 3));
                 }
+            // the next tile goes to the other buffer while this tile's fragments are on their way from LDS
+            if (key0 + BN < keys_scored) stage(cur ^ 1);
             float16_t sc[2][2];
             const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -701,6 +678,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
 #pragma unroll
                 for (int c = 0; c < 2; c++)   // cbsz = blgp = 1: both operands are BF8 (E5M2); no block scales
                     sc[b][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[c], qf[b], zero16, 1, 1, 0, 0, 0, 0);
+            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);   // the tile after that into registers
 #pragma unroll
             for (int b = 0; b < 2; b++) {
                 // ---- online softmax of one 32-query block; p = 2^(s * c - m * c) on the raw-score maximum
@@ -759,6 +737,10 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
             }
         }
         __syncthreads();  // tile i+1 is visible; every wave is done reading tile i
+    };
+    for (int key0 = 0; key0 < keys_scored; key0 += 2 * BN) {
+        tile_body(key0, std::integral_constant<int, 0>{});
+        if (key0 + BN < keys_scored) tile_body(key0 + BN, std::integral_constant<int, 1>{});
     }
 
     // ---- epilogue: the two lanes of a query add their shares of the row sum; normalise, store [q][dd]
@@ -859,12 +841,13 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
         case 64:   // all four query blocks of a wave share every K fragment
             // eight waves halve the staging work per query (-2 % time); a causal tile of 512 queries
             // would idle its early waves through too many masked key tiles
-            if constexpr (MODE == FEATHER_E5M2) if (!getenv("FEATHER_EXP_ATTN64_OLD")) {   // the FP8-rate kernel, same two workgroup shapes
+            if constexpr (MODE == FEATHER_E5M2) {   // the FP8-rate kernel, same two workgroup shapes
                 if (!a.causal && fills_chip(512)) return launch_attn64_bf8<VC, 8, 1>(a, s);
                 return launch_attn64_bf8<VC, 4, 2>(a, s);
+            } else {
+                if (!a.causal && fills_chip(512)) return launch_attn<64, MODE, 4, 4, 64, 1, VC, 8>(a, s);
+                return launch_attn<64, MODE, 4, 4, 64, 2, VC>(a, s);
             }
-            if (!a.causal && fills_chip(512)) return launch_attn<64, MODE, 4, 4, 64, 1, VC, 8>(a, s);
-            return launch_attn<64, MODE, 4, 4, 64, 2, VC>(a, s);
         case 128:
             if (fills_chip(256)) return launch_attn<128, MODE, 2, 2, 64, 1, VC, 8>(a, s);
             return launch_attn<128, MODE, 2, 2, 64, 2, VC>(a, s);

@@ -499,14 +499,15 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef int int8v_t __attribute__((ext_vector_type(8)));
 
-template <bool VC, int WAVES, int OCC>
-__global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
+template <int MODE, bool VC, int WAVES, int OCC>
+__global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
     const uint32_t *__restrict__ q, const uint32_t *__restrict__ k, const uint32_t *__restrict__ v,
     float *__restrict__ out, int L, int n_heads, int kv_group, int tiles_per_head, float scale_log2e,
     int keys_scored, int mask_tail, const int32_t *__restrict__ cu_seqlens, int tiles_per_seq, int total_rows,
     int causal) {
     constexpr int D = 64, DW = 16, BN = 64;
-    constexpr int KP = D + 16;             // K row pitch in LDS, bytes
+    constexpr bool BF8 = MODE == FEATHER_E5M2;   // K and Q stay packed bytes; otherwise both are decoded to fp16
+    constexpr int KP = (BF8 ? D : 2 * D) + 16;   // K row pitch in LDS, bytes
     constexpr int VS = BN;                 // fp16 per V^T row
     constexpr int kThreads = 64 * WAVES, QT = 64 * WAVES;
     constexpr int UNITS = BN * D / 16;     // 16-code units of a K (or V) tile: 256
@@ -547,18 +548,29 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
     const uint32_t *kh = k + kv_row0 * DW;
     const uint32_t *vh = v + kv_row0 * DW;
 
-    // ---- Q operands: 32 bytes of the lane's query row per 32-query block
-    int8v_t qf[2];
+    // ---- Q operands per 32-query block: 32 bytes of the lane's query row (bf8), or four fp16 fragments of the
+    // eight dims 16 st + 8 h .. + 7 (the k-slots of this lane in the st-th 32x32x16 step)
+    int8v_t qf[BF8 ? 2 : 1];
+    half8_t qh16[BF8 ? 1 : 2][BF8 ? 1 : 4];
 #pragma unroll
     for (int b = 0; b < 2; b++) {
         const int row = q0 + 32 * b + n;
-        u32x4 w0 = u32x4{0, 0, 0, 0}, w1 = u32x4{0, 0, 0, 0};
-        if (row < L) {
-            const u32x4 *src = reinterpret_cast<const u32x4 *>(qh + (int64_t)row * DW + 8 * h);
-            w0 = src[0];
-            w1 = src[1];
+        if constexpr (BF8) {
+            u32x4 w0 = u32x4{0, 0, 0, 0}, w1 = u32x4{0, 0, 0, 0};
+            if (row < L) {
+                const u32x4 *src = reinterpret_cast<const u32x4 *>(qh + (int64_t)row * DW + 8 * h);
+                w0 = src[0];
+                w1 = src[1];
+            }
+            qf[b] = int8v_t{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+        } else {
+#pragma unroll
+            for (int st = 0; st < 4; st++) {
+                u32x2 w = u32x2{0, 0};
+                if (row < L) w = *reinterpret_cast<const u32x2 *>(qh + (int64_t)row * DW + 4 * st + 2 * h);
+                qh16[b][st] = dec8<MODE>(w.x, w.y);
+            }
         }
-        qf[b] = int8v_t{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
     }
 
     constexpr float kLazy = 8.f;
@@ -615,20 +627,40 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
         _Float16 *vt_lds = reinterpret_cast<_Float16 *>(k_lds + BN * KP);
         if (stages_k) {
             const int key = kt_id / 4, c16 = kt_id % 4;
-            *reinterpret_cast<u32x4 *>(k_lds + key * KP + 16 * c16) = kreg;
+            if constexpr (BF8) {
+                *reinterpret_cast<u32x4 *>(k_lds + key * KP + 16 * c16) = kreg;
+            } else {
+                half8_t *kd = reinterpret_cast<half8_t *>(k_lds + key * KP + 32 * c16);
+                kd[0] = dec8<MODE>(kreg.x, kreg.y);
+                kd[1] = dec8<MODE>(kreg.z, kreg.w);
+            }
         }
         if (stages_v) {
             // V: 4 keys x 4 dims -> V^T[dd][slot]; keys 4 kg .. 4 kg + 3 are quarter q4 = kg % 4 of their group of
             // 16 and go to slots 8 (q4 & 1) + 4 (q4 >> 1) .. + 3 of it
             const int ddw = tid % DW, kg = tid / DW;
             const int q4 = kg & 3, pos = 16 * (kg >> 2) + 8 * (q4 & 1) + 4 * (q4 >> 1);
+            uint32_t lo2[4], hi2[4];   // halfs (key 0, key 1) and (key 2, key 3) of dim 4 ddw + c
+            if constexpr (BF8) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) {   // byte c of each word, placed as the high byte of its half
+                    const uint32_t sel = 0x000c000cu | ((uint32_t)c << 8) | ((uint32_t)(4 + c) << 24);
+                    lo2[c] = perm(vreg[1], vreg[0], sel);
+                    hi2[c] = perm(vreg[3], vreg[2], sel);
+                }
+            } else {
+                uint32_t p01[4], p23[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) dec_word<MODE>(vreg[r], p01[r], p23[r]);
+                lo2[0] = perm(p01[1], p01[0], 0x05040100u); hi2[0] = perm(p01[3], p01[2], 0x05040100u);
+                lo2[1] = perm(p01[1], p01[0], 0x07060302u); hi2[1] = perm(p01[3], p01[2], 0x07060302u);
+                lo2[2] = perm(p23[1], p23[0], 0x05040100u); hi2[2] = perm(p23[3], p23[2], 0x05040100u);
+                lo2[3] = perm(p23[1], p23[0], 0x07060302u); hi2[3] = perm(p23[3], p23[2], 0x07060302u);
+            }
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                // halfs (key r, key r + 1) of dim 4 ddw + c: byte c of each word, placed as the high byte
-                const uint32_t sel = 0x000c000cu | ((uint32_t)c << 8) | ((uint32_t)(4 + c) << 24);
-                const uint32_t lo2 = perm(vreg[1], vreg[0], sel), hi2 = perm(vreg[3], vreg[2], sel);
                 const int row = 4 * ddw + c;
-                *reinterpret_cast<u32x2 *>(vt_lds + row * VS + (((pos >> 3) ^ swz(row)) << 3) + (pos & 4)) = u32x2{lo2, hi2};
+                *reinterpret_cast<u32x2 *>(vt_lds + row * VS + (((pos >> 3) ^ swz(row)) << 3) + (pos & 4)) = u32x2{lo2[c], hi2[c]};
             }
         }
     };
@@ -649,17 +681,20 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
             diag = causal && key0 + BN - 1 > q0;          // some key of the tile lies past the wave's first query
             skip = causal && key0 > q0 + 63;              // every key lies past the wave's last query
         }
-        if (skip) {   // nothing to score for this wave; the other waves still need the next tile
+        if constexpr (VC) {   // a wave with nothing to score in this tile still stages: one copy of that code, up front
             if (key0 + BN < keys_scored) stage(cur ^ 1);
             if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
-        } else {
+        }
+        if (!skip) {
             // ---- S^T = K Q^T, raw scores: [query block][key block]
-            int8v_t kf[2];
+            int8v_t kf[BF8 ? 2 : 1];
+            if constexpr (BF8) {
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const u32x4 *src = reinterpret_cast<const u32x4 *>(k_lds + (32 * c + n) * KP + 32 * h);
-                const u32x4 w0 = src[0], w1 = src[1];
-                kf[c] = int8v_t{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+                for (int c = 0; c < 2; c++) {
+                    const u32x4 *src = reinterpret_cast<const u32x4 *>(k_lds + (32 * c + n) * KP + 32 * h);
+                    const u32x4 w0 = src[0], w1 = src[1];
+                    kf[c] = int8v_t{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+                }
             }
             half8_t vf[4][2];   // [16-key step][32-dim block]
 #pragma unroll
@@ -670,15 +705,30 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_bf8_kernel(
                     vf[g][d] = *reinterpret_cast<const half8_t *>(vt_lds + row * VS + (((2 * g + h) ^ swz(row)) << 3));
                 }
             // the next tile goes to the other buffer while this tile's fragments are on their way from LDS
-            if (key0 + BN < keys_scored) stage(cur ^ 1);
+            if constexpr (!VC) if (key0 + BN < keys_scored) stage(cur ^ 1);
             float16_t sc[2][2];
             const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if constexpr (BF8) {
 #pragma unroll
-            for (int b = 0; b < 2; b++)
+                for (int b = 0; b < 2; b++)
 #pragma unroll
-                for (int c = 0; c < 2; c++)   // cbsz = blgp = 1: both operands are BF8 (E5M2); no block scales
-                    sc[b][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[c], qf[b], zero16, 1, 1, 0, 0, 0, 0);
-            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);   // the tile after that into registers
+                    for (int c = 0; c < 2; c++)   // cbsz = blgp = 1: both operands are BF8 (E5M2); no block scales
+                        sc[b][c] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[c], qf[b], zero16, 1, 1, 0, 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 2; c++) {   // one key block at a time: four fp16 K fragments live
+                    half8_t k16[4];
+#pragma unroll
+                    for (int st = 0; st < 4; st++)
+                        k16[st] = *reinterpret_cast<const half8_t *>(k_lds + (32 * c + n) * KP + 32 * st + 16 * h);
+#pragma unroll
+                    for (int b = 0; b < 2; b++)
+#pragma unroll
+                        for (int st = 0; st < 4; st++)
+                            sc[b][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(k16[st], qh16[b][st], st == 0 ? zero16 : sc[b][c], 0, 0, 0);
+                }
+            }
+            if constexpr (!VC) if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);   // the tile after that into registers
 #pragma unroll
             for (int b = 0; b < 2; b++) {
                 // ---- online softmax of one 32-query block; p = 2^(s * c - m * c) on the raw-score maximum
@@ -802,10 +852,10 @@ static int launch_attn(const AttnArgs &a, hipStream_t s) {
     return check_launch("feather_flash_attn_fp8");
 }
 
-template <bool VC, int WAVES, int OCC>
-static int launch_attn64_bf8(const AttnArgs &a, hipStream_t s) {
+template <int MODE, bool VC, int WAVES, int OCC>
+static int launch_attn64_wide(const AttnArgs &a, hipStream_t s) {
     constexpr int QT = 64 * WAVES, BN = 64, D = 64;
-    constexpr size_t lds = (size_t)(BN * (D + 16) + D * BN * 2) * 2;   // two (K bytes, V^T fp16) buffers
+    constexpr size_t lds = (size_t)(BN * ((MODE == FEATHER_E5M2 ? D : 2 * D) + 16) + D * BN * 2) * 2;   // two (K, V^T fp16) buffers
     const int64_t L = VC ? a.max_seqlen : a.L;
     const int tiles_per_seq = (int)((L + QT - 1) / QT);
     const int64_t tiles = VC ? tiles_per_seq * a.n_seq : tiles_per_seq;
@@ -815,7 +865,7 @@ static int launch_attn64_bf8(const AttnArgs &a, hipStream_t s) {
     // both tail modes score whole 64-key tiles here (the reference scores zero rows past L, the mask hides them)
     const int64_t keys_scored = (L + BN - 1) / BN * BN;
     const float log2e = 1.4426950408889634f;
-    hipLaunchKernelGGL((flash_attn64_bf8_kernel<VC, WAVES, OCC>), dim3((unsigned)blocks), dim3(64 * WAVES), lds, s,
+    hipLaunchKernelGGL((flash_attn64_wide_kernel<MODE, VC, WAVES, OCC>), dim3((unsigned)blocks), dim3(64 * WAVES), lds, s,
                        (const uint32_t *)a.q, (const uint32_t *)a.k, (const uint32_t *)a.v, (float *)a.out, (int)L,
                        (int)a.n_heads, (int)a.kv_group, (int)tiles, a.scale * log2e, (int)keys_scored,
                        a.tail == FEATHER_TAIL_MASK ? 1 : 0, (const int32_t *)a.cu_seqlens, tiles_per_seq,
@@ -841,13 +891,8 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
         case 64:   // all four query blocks of a wave share every K fragment
             // eight waves halve the staging work per query (-2 % time); a causal tile of 512 queries
             // would idle its early waves through too many masked key tiles
-            if constexpr (MODE == FEATHER_E5M2) {   // the FP8-rate kernel, same two workgroup shapes
-                if (!a.causal && fills_chip(512)) return launch_attn64_bf8<VC, 8, 1>(a, s);
-                return launch_attn64_bf8<VC, 4, 2>(a, s);
-            } else {
-                if (!a.causal && fills_chip(512)) return launch_attn<64, MODE, 4, 4, 64, 1, VC, 8>(a, s);
-                return launch_attn<64, MODE, 4, 4, 64, 2, VC>(a, s);
-            }
+            if (!a.causal && fills_chip(512)) return launch_attn64_wide<MODE, VC, 8, 1>(a, s);
+            return launch_attn64_wide<MODE, VC, 4, 2>(a, s);
         case 128:
             if (fills_chip(256)) return launch_attn<128, MODE, 2, 2, 64, 1, VC, 8>(a, s);
             return launch_attn<128, MODE, 2, 2, 64, 2, VC>(a, s);

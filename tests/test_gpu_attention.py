@@ -109,6 +109,39 @@ def test_flash_attention_invariants_and_gqa(dev, orc):
     assert torch.equal(grouped, rep)
 
 
+@pytest.mark.parametrize("mode", ["E5M2", "E4M3"])
+@pytest.mark.parametrize("d", [64, 128, 256, 512])
+@pytest.mark.parametrize("ramp", ["steps", "creep", "fall"])
+def test_flash_attention_rising_scores(dev, orc, mode, d, ramp):
+    """The kernels raise the reference point of their exponentials lazily (only when a score exceeds it by
+    more than 2^8): scores that jump by ~2^30 every 48 keys (inside and across key tiles), that creep up by
+    a few binary orders per tile, or that start at their maximum and fall, must all give the closed-form
+    softmax (float64, of the decoded operands)."""
+    from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
+    rng = np.random.default_rng(d + len(ramp))
+    heads, L = 2, 400
+    j = np.arange(L, dtype=np.float64)
+    c = 1.4426950408889634 / np.sqrt(d)                # exponent units per raw score unit
+    if ramp == "steps":
+        lift = np.floor(j / 48) * 30.0                 # binary orders of magnitude
+    elif ramp == "creep":
+        lift = j * (5.0 / 64)
+    else:
+        lift = (L - j) * (20.0 / 64)
+    # q = 0.5 in every dim (+ noise), k_j = kval_j in every dim (+ noise): raw score ~ d * 0.5 * kval_j
+    kval = lift / c / (0.5 * d)
+    q = (0.5 + 0.05 * rng.standard_normal((heads, L, d))).astype(np.float16)
+    k = (kval[None, :, None] + 0.05 * rng.standard_normal((heads, L, d))).astype(np.float16)
+    v = rng.standard_normal((heads, L, d)).astype(np.float16)
+    qp, kp, vp = (orc.pack_fp8(a, mode) for a in (q, k, v))
+    out = flash_attention_fp8_acc_fp32_gpu(_dev_words(qp, dev), _dev_words(kp, dev), _dev_words(vp, dev), L, d // 4,
+                                           mode=mode)
+    got = out.cpu().numpy().reshape(heads, L, d)
+    assert np.isfinite(got).all()
+    want64 = orc.attention_f64_np(qp, kp, vp, L, d, mode)
+    assert _nerr(got, want64) <= TOL
+
+
 @pytest.mark.parametrize("d", [64, 128])
 def test_flash_attention_e5m2_subnormal_codes_count(dev, orc, d):
     """E5M2 scores must keep subnormal codes exact: keys of code 0x01 (2^-16) against queries of

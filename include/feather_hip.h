@@ -249,9 +249,9 @@ int64_t feather_decode_step_scratch_bytes(const feather_decoder_t *dec, int64_t 
 
 /* token_ids [batch] int32, block_tables [batch, max_blocks] int32, ctx_lens [batch] int32 (tokens
  * already in the cache; the caller adds 1 after the step), logits [batch, vocab] fp32.
- * batch <= 64; max_ctx bounds ctx_lens + 1.
- * seq_status [batch] int32 or NULL: 0 = the new token's K/V were appended; 1 = ctx_lens[b] is negative
- * or the block table is full (>= max_blocks * block_size); 2 = the table entry of the new position is
+ * batch <= 64; max_ctx (<= max_blocks * block_size) bounds ctx_lens + 1.
+ * seq_status [batch] int32 or NULL: 0 = the new token's K/V were appended; 1 = the new position
+ * ctx_lens[b] is negative or not below max_ctx (no room for it); 2 = the table entry of the new position is
  * not a block of the cache (outside [0, n_blocks)).  With 1 or 2 nothing is written to the cache for
  * that sequence and its logits come from the tokens already cached: the caller must not use them. */
 int feather_decode_step(const feather_decoder_t *dec, const void *token_ids, const void *block_tables,

@@ -1,6 +1,10 @@
 // Flash-attention forward on FP8-packed Q/K/V (prefill): fixed-length heads, or variable-length
 // sequences packed back to back with an optional causal mask.
 //
+// Two kernels: flash_attn_kernel (this comment; head dims 128, 256, 512) on the 16x16x32 matrix
+// instructions, and flash_attn64_wide_kernel (head dim 64, further down) on the 32x32 ones, which
+// shares the work split, the staging scheme and the numerics and documents what differs.
+//
 // Work split.  One workgroup (WAVES waves, 4 or 8) owns a tile of 16*QB*WAVES/KSPLIT
 // queries of one head; each wave owns 16*QB of them for the whole key loop (with KSPLIT = 2 two
 // waves share them and each scores one half of the keys of every tile).  Keys/values are
@@ -34,7 +38,9 @@
 // softmax in fp32 (computed as 2^x with log2(e) folded into the scale), P
 // rounded to fp16 before P.V, fp32 output.  One difference inside the stated
 // tolerance: the denominator sums the fp16-rounded P (the values that multiply
-// V) where the reference sums P before rounding.
+// V) where the reference sums P before rounding.  The point the exponentials
+// refer to is a running maximum that is raised lazily (see softmax_block): the
+// quotient O / l does not depend on it.
 #include <type_traits>
 #include "common.h"
 

@@ -142,6 +142,61 @@ def test_flash_attention_rising_scores(dev, orc, mode, d, ramp):
     assert _nerr(got, want64) <= TOL
 
 
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_flash_attention_e4m3_kernel_decode_codes(dev, orc, d):
+    """E4M3 operands are decoded as the reference kernel does (gemv.py:83-88), not as OCP FP8: a zero-exponent
+    code c is m * 2^-17 (OCP: m * 2^-9) and 0x7F / 0xFF are +-480 (OCP: NaN).  Keys made of 0x7F against keys
+    made of 0x7E (448) and of zero-exponent codes: an OCP decode would give NaN, and 256 x larger scores for
+    the zero-exponent keys."""
+    from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
+    rng = np.random.default_rng(d)
+    L = 192
+    K = np.zeros((L, d), np.uint8)
+    K[0::3] = 0x7F                                     # 480 in every dim
+    K[1::3] = 0x7E                                     # 448
+    K[2::3] = rng.integers(1, 8, size=(L // 3, d))     # zero-exponent codes 0x01..0x07
+    Q = np.full((L, d), 0x18, np.uint8)                # 2^-4: raw scores 30 d, 28 d and ~0
+    Q[1::2] = 0x98                                     # and -2^-4 for the odd queries
+    V = rng.integers(0x30, 0x48, size=(L, d)).astype(np.uint8)   # values around 1
+    V[0::3] |= 0x80
+    q, k, v = (np.ascontiguousarray(a).view(np.uint32) for a in (Q, K, V))
+    out = flash_attention_fp8_acc_fp32_gpu(_dev_words(q, dev), _dev_words(k, dev), _dev_words(v, dev), L, d // 4,
+                                           mode="E4M3").cpu().numpy()
+    assert np.isfinite(out).all()
+    want = orc.attention_f64_np(q, k, v, L, d, "E4M3")[0]
+    assert _nerr(out, want) <= TOL
+    # even queries attend to the 480-keys (negative V), odd queries to the zero-exponent keys (scores ~0 against
+    # -30 d and -28 d): the two groups of rows must differ the way the closed form says
+    assert want[0].mean() < 0 < want[1].mean()
+
+
+def test_flash_attention_repeatable_and_graph_replay(dev, orc):
+    """Same inputs, same bits: across calls and across replays of a captured HIP graph (the kernels hold no state
+    between calls and have no atomics)."""
+    from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
+    import feather_amd as feather
+    g = torch.Generator(device=dev).manual_seed(7)
+    for mode, H, L, d in (("E5M2", 8, 1024, 64), ("E4M3", 8, 1024, 64), ("E4M3", 2, 512, 256)):
+        qkv = [feather.pack_fp8_tensor(torch.randn(H, L, d, generator=g, device=dev).half(), mode=mode).view(H, L, d // 4)
+               for _ in range(3)]
+        ref = flash_attention_fp8_acc_fp32_gpu(*qkv, L, d // 4, mode=mode).clone()
+        again = flash_attention_fp8_acc_fp32_gpu(*qkv, L, d // 4, mode=mode)
+        assert torch.equal(ref, again)
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            flash_attention_fp8_acc_fp32_gpu(*qkv, L, d // 4, mode=mode)
+        torch.cuda.current_stream().wait_stream(s)
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            out = flash_attention_fp8_acc_fp32_gpu(*qkv, L, d // 4, mode=mode)
+        for _ in range(3):
+            out.zero_()
+            gr.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, ref)
+
+
 @pytest.mark.parametrize("d", [64, 128])
 def test_flash_attention_e5m2_subnormal_codes_count(dev, orc, d):
     """E5M2 scores must keep subnormal codes exact: keys of code 0x01 (2^-16) against queries of

@@ -213,7 +213,7 @@ def main() -> int:
     ttab = load_traffic()
     headline = roofline_record(ttab, "gemv_e4m3_16384", "gemv_fp8_kernel<E4M3>", gemv_bytes, kern_us)
 
-    extra = {"gemv_e4m3_16384_cold_first_series_us": round(cold_us, 2)}   # same kernel before the clocks are up
+    extra = {"gemv_e4m3_16384_cold_first_series_us": round(cold_us, 2)}   # same kernel, first series: no warm-up, first-launch cost included
     rl = {}                                                               # roofline records of the other HBM-bound workloads
     if not args.no_extra:
         # cache-resident figure (one matrix re-used): reported separately, never the headline

@@ -93,13 +93,14 @@ __device__ __forceinline__ void dec_e5m2_word(uint32_t w, uint32_t &p01, uint32_
 
 // E4M3 code -> fp16 bits sign | (e ? e + 8 : 0) << 10 | m << 7 (reference
 // gemv.py:83-88), four codes at a time with byte-parallel integer arithmetic:
-//   high byte  H = sign | u + (e > 0 ? 0x20 : 0),  u = (c >> 1) & 0x3F = e << 2 | m >> 1
+//   high byte  H = sign | (a + (e > 0 ? 0x40 : 0)) >> 1,  a = c & 0x7F = e << 3 | m
 //   low byte   L = (c & 1) << 7
-// (e > 0) is (u >= 4), bit 7 of u + 0x7C; no byte ever carries into the next.
+// (e > 0) is (a >= 8), bit 7 of a + 0x78.  v_lerp_u8 computes (x + y + (z & 1)) >> 1 on each byte with a 9-bit
+// intermediate, i.e. an add and a shift in one instruction and no carry between bytes.
 __device__ __forceinline__ void dec_e4m3_word(uint32_t w, uint32_t &p01, uint32_t &p23) {
-    uint32_t u = (w >> 1) & 0x3F3F3F3Fu;
-    uint32_t bias = ((u + 0x7C7C7C7Cu) >> 2) & 0x20202020u;
-    uint32_t hi = (w & 0x80808080u) | (u + bias);
+    uint32_t a = w & 0x7F7F7F7Fu;
+    uint32_t bias = __builtin_amdgcn_lerp(a, 0x78787878u, 0u) & 0x40404040u;
+    uint32_t hi = (w & 0x80808080u) | __builtin_amdgcn_lerp(a, bias, 0u);
     uint32_t lo = (w << 7) & 0x80808080u;
     p01 = perm(hi, lo, 0x05010400u);
     p23 = perm(hi, lo, 0x07030602u);

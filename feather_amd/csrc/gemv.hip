@@ -56,6 +56,27 @@ constexpr int kGemvWaves = kGemvThreads / kWave;
 constexpr int kMaxChunk = 32768;  // codes of the vector held in LDS at once (64 KiB as fp16)
 
 // 16 codes (one uint4) of a row against the matching 16 fp16 of the vector.
+// Keeps a wave-uniform value in scalar registers, so that the compiler does not fold it into per-lane
+// (vector) address arithmetic.
+__device__ __forceinline__ uint32_t pin_scalar(uint32_t v) {
+    asm volatile("" : "+s"(v));
+    return v;
+}
+// Same for a per-lane 32-bit offset: pinned next to its use, its zero extension stays in the block of the load
+// and the load takes the form "scalar 64-bit base + 32-bit vector offset".
+__device__ __forceinline__ uint32_t pin_vector(uint32_t v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+typedef const __attribute__((address_space(1))) uint8_t *global_u8_ptr;   // global address space kept through the asm
+__device__ __forceinline__ global_u8_ptr pin_scalar(global_u8_ptr p) {
+    asm volatile("" : "+s"(p));
+    return p;
+}
+__device__ __forceinline__ u32x4 load_nt128_global(global_u8_ptr p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x4 *>(p));
+}
+
 template <int MODE>
 __device__ __forceinline__ float mac16(const u32x4 &a, const u32x4 &x0, const u32x4 &x1, float acc) {
     uint32_t p, q;
@@ -108,6 +129,7 @@ __global__ __launch_bounds__(WAVES * kWave) void gemv_fp8_kernel(const uint8_t *
     u32x4 a[RPW][U];
     auto issue = [&](int r0, int it) {
         const int s0 = (int)(((unsigned)(r0 / RPW) * (unsigned)kStagger) % (unsigned)n_steps);
+        const uint32_t lane_off = pin_vector((uint32_t)(lane * 16));
 #pragma unroll
         for (int u = 0; u < U; u++) {
             int st = it + u + s0;
@@ -116,8 +138,9 @@ __global__ __launch_bounds__(WAVES * kWave) void gemv_fp8_kernel(const uint8_t *
 #pragma unroll
             for (int r = 0; r < RPW; r++) {
                 const int row = min(r0 + r, M - 1);  // surplus rows re-read the last row, result dropped
-                if (FULL || col[u] + lane * 16 < kc)
-                    a[r][u] = load_nt128(m + (int64_t)row * K + k0 + lane * 16 + col[u]);
+                // wave-uniform 64-bit base (scalar registers) + the lane's 32-bit offset: no vector address arithmetic
+                global_u8_ptr base = pin_scalar((global_u8_ptr)(m + (int64_t)row * K + k0 + col[u]));
+                if (FULL || col[u] + lane * 16 < kc) a[r][u] = load_nt128_global(base + lane_off);
                 else a[r][u] = u32x4{0, 0, 0, 0};
             }
         }
@@ -178,8 +201,10 @@ __global__ __launch_bounds__(WAVES * kWave) void gemv_fp8_kernel(const uint8_t *
             have = false;
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                int c8 = (col[u] + lane * 16) / 8;
-                u32x4 x0 = lds128[c8], x1 = lds128[c8 + 1];
+                // fp16 vector: 2 bytes per column; scalar step offset + the lane's constant offset
+                const u32x4 *xp = reinterpret_cast<const u32x4 *>(reinterpret_cast<const uint8_t *>(lds32) +
+                                                                  pin_scalar(2u * (uint32_t)col[u]) + (uint32_t)(lane * 32));
+                u32x4 x0 = xp[0], x1 = xp[1];
 #pragma unroll
                 for (int r = 0; r < RPW; r++) acc[r] = mac16<MODE>(a[r][u], x0, x1, acc[r]);
             }

@@ -73,14 +73,14 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
     const int c_begin = blockIdx.y * cps, c_end = min(c_begin + cps, n_chunks);
     const uint8_t *wp = w + (int64_t)row * K + 16 * kb;
     // this thread's share of the vectors' chunk: 16-byte piece (vec, col16) = (piece / 16, piece % 16)
+    // (columns of vectors past nvec are filled from the last vector: their sums are never stored, and a column of
+    // the MFMA result depends on its own vector only, so the loads need no lane mask)
     const uint8_t *xp[NB];
-    bool xok[NB];
     int xdst[NB];
 #pragma unroll
     for (int i = 0; i < NB; i++) {
         int piece = tig + kBgThreads * i;
         int vec = piece >> 4, col16 = piece & 15;
-        xok[i] = vec < nvec;
         xp[i] = x + (int64_t)min(vec, nvec - 1) * K + 16 * col16;
         xdst[i] = vec * kBgPitch + 16 * col16;
     }
@@ -94,7 +94,7 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
 #pragma unroll
         for (int u = 0; u < 4; u++) wr[u] = *reinterpret_cast<const u32x4 *>(wp + col + 64 * u);
 #pragma unroll
-        for (int i = 0; i < NB; i++) xr[i] = xok[i] ? *reinterpret_cast<const u32x4 *>(xp[i] + col) : u32x4{0, 0, 0, 0};
+        for (int i = 0; i < NB; i++) xr[i] = *reinterpret_cast<const u32x4 *>(xp[i] + col);
     };
     // One chunk: vectors' chunk -> LDS, (the caller's prefetch goes here), barrier, MFMAs.
     auto stage_x = [&](int it, const u32x4 (&xr)[NB]) {
@@ -134,21 +134,29 @@ __global__ __launch_bounds__(kBgThreads * KG) void gemv_batched_kernel(const uin
     // Every chunk but the last prefetches its successor unconditionally, so the number of loads
     // in flight is known at compile time and the wait for chunk c leaves chunk c + 1 outstanding
     // (a prefetch inside an `if` makes the compiler wait for everything).
-    for (int it = grp; it < n_it - KG; it += KG) {
-        const _Float16 *buf = stage_x(it, xa);
-        u32x4 wn[4], xn[NB];
+    // The loop is unrolled by two so that the two register sets swap roles without copies.
+    u32x4 wb[4], xb[NB];
+    auto step = [&](int it, const u32x4 (&wc)[4], const u32x4 (&xc)[NB], u32x4 (&wn)[4], u32x4 (&xn)[NB]) {
+        const _Float16 *buf = stage_x(it, xc);
         issue(chunk_of(it + KG), wn, xn);
         __syncthreads();
-        mac(buf, wa);
-#pragma unroll
-        for (int u = 0; u < 4; u++) wa[u] = wn[u];
-#pragma unroll
-        for (int i = 0; i < NB; i++) xa[i] = xn[i];
-    }
-    {
-        const _Float16 *buf = stage_x(n_it - KG + grp, xa);
+        mac(buf, wc);
+    };
+    auto last = [&](const u32x4 (&wc)[4], const u32x4 (&xc)[NB]) {
+        const _Float16 *buf = stage_x(n_it - KG + grp, xc);
         __syncthreads();
-        mac(buf, wa);
+        mac(buf, wc);
+    };
+    int it = grp;
+    for (; it + KG < n_it - KG; it += 2 * KG) {
+        step(it, wa, xa, wb, xb);
+        step(it + KG, wb, xb, wa, xa);
+    }
+    if (it < n_it - KG) {
+        step(it, wa, xa, wb, xb);
+        last(wb, xb);
+    } else {
+        last(wa, xa);
     }
     if constexpr (KG > 1) {
         // groups 1.. -> group 0 through LDS (the vectors' buffers are free once every wave is past its MFMAs)

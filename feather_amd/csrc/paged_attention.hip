@@ -59,13 +59,10 @@ __device__ __forceinline__ void v_pairs(uint32_t wa, uint32_t wb, uint32_t out[4
         for (int c = 0; c < 4; c++)
             out[c] = perm(wb, wa, 0x000c000cu | ((uint32_t)c << 8) | ((uint32_t)(4 + c) << 24));
     } else {
-        uint32_t a01, a23, b01, b23;
-        dec_word<MODE>(wa, a01, a23);
-        dec_word<MODE>(wb, b01, b23);
-        out[0] = perm(b01, a01, 0x05040100u);
-        out[1] = perm(b01, a01, 0x07060302u);
-        out[2] = perm(b23, a23, 0x05040100u);
-        out[3] = perm(b23, a23, 0x07060302u);
+        // interleave the codes of the two tokens first ((a0 b0 a1 b1), (a2 b2 a3 b3)): the decoder's own
+        // pairs are then the (tok a, tok b) pairs
+        dec_word<MODE>(perm(wb, wa, 0x05010400u), out[0], out[1]);
+        dec_word<MODE>(perm(wb, wa, 0x07030602u), out[2], out[3]);
     }
 }
 

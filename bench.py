@@ -29,11 +29,13 @@ MFMA_PEAK_F16_TFLOPS = 2500.0  # dense fp16/bf16, published
 WARM_MS = 40.0                  # warm-up time of the attention series (ours and SDPA alike)
 
 
-def gpu_time_us(fn, steps, warmup, sync, warm_ms=0.0):
+def gpu_time_us(fn, steps, warmup, sync, warm_ms=0.0, gate=3):
     """Average microseconds per call over `steps` back-to-back calls (HIP events on the
     stream the kernels are launched on: torch's current stream).  With `warm_ms` the warm-up calls are
     repeated until that many milliseconds of back-to-back work have passed: the first tens of
-    milliseconds of a series run below the sustained clock."""
+    milliseconds of a series run below the sustained clock.  `gate` untimed calls right after the last
+    synchronize keep the device busy while the host enqueues the start event and the first timed calls
+    (otherwise the host's per-call cost before the first launch is counted as kernel time)."""
     import torch
     t0 = time.perf_counter()
     for i in range(warmup):
@@ -44,9 +46,11 @@ def gpu_time_us(fn, steps, warmup, sync, warm_ms=0.0):
             fn(i)
         sync()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(gate):
+        fn(i)
     start.record()
     for i in range(steps):
-        fn(i)
+        fn(gate + i)
     stop.record()
     sync()
     return start.elapsed_time(stop) * 1000.0 / steps
@@ -182,24 +186,32 @@ def main() -> int:
     # run for ~50 ms before the W warm-up steps; the timed region stays exactly K steps.
     PREWARM = args.prewarm
     sync()
-    cold_us = gpu_time_us(gemv_step("E4M3"), args.steps, 0, sync)   # the first series of the process, no warm-up at all
+    cold_us = gpu_time_us(gemv_step("E4M3"), args.steps, 0, sync, gate=0)   # the first series of the process, no warm-up at all
     for i in range(PREWARM):
         gemv_step("E4M3")(i)
     # the whole timed region, bracketed by synchronize on both sides
     for i in range(args.warmup):
         gemv_step("E4M3")(i)
     sync()
+    # After a synchronize the queue is empty: the first launch reaches the device only after the host's
+    # per-call cost (~15 us of wrapper and dispatch), which HIP events around K launches would count as
+    # kernel time (0.7 us per launch at K = 20).  GATE untimed launches of the same kernel keep the device
+    # busy while the host enqueues the start event and the first timed launches, so the events enclose
+    # exactly K back-to-back launches; the wall clock covers all GATE + K launches.
+    GATE = 3
     t0 = time.perf_counter()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    ev0.record()
     step = gemv_step("E4M3")
+    for i in range(GATE):
+        step(args.warmup + i)
+    ev0.record()
     for i in range(args.steps):
-        step(i)
+        step(args.warmup + GATE + i)
     ev1.record()
     sync()
     wall_ms = (time.perf_counter() - t0) * 1000.0
     kern_us = ev0.elapsed_time(ev1) * 1000.0 / args.steps
-    ms_per_step = wall_ms / args.steps
+    ms_per_step = wall_ms / (args.steps + GATE)
 
     if args.calibrate_copy:
         src = torch.empty(M * K // 4, dtype=torch.int32, device=dev).fill_(1)
@@ -418,7 +430,7 @@ def main() -> int:
         "config": {"workload": "E4M3 packed GEMV 16384x16384 + vector 16384 (the configuration the metric is quoted on); N(0,1) fp16 "
                                "sources with 1% of entries x1e-3, packed 4 codes per 32-bit word; 4 distinct "
                                "matrices (1 GiB) rotated",
-                   "M": M, "K": K, "mode": "E4M3", "buffers": NBUF, "clock_prewarm_launches": PREWARM},
+                   "M": M, "K": K, "mode": "E4M3", "buffers": NBUF, "clock_prewarm_launches": PREWARM, "gate_launches": GATE},
         "roofline": dict(headline, avg_launch_us=round(kern_us, 3)),
         "cpu_baseline": cpu,
         "extra": dict(extra, roofline=rl),

@@ -103,7 +103,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     // a tile with fewer units than threads is staged by the first UNITS threads (whole waves)
     constexpr bool ALL_STAGE = UNITS >= kAttnThreads;
     static_assert(UNITS % 64 == 0 && (ALL_STAGE ? UNITS % kAttnThreads == 0 : true), "tile / workgroup mismatch");
-    constexpr int KB16 = BN / 16, KB32 = BN / 32, DB = D / 16, STEPS = D / 32;
+    constexpr int DB = D / 16, STEPS = D / 32;
     constexpr int GBN = BN / KSPLIT;       // keys of a tile that one key group scores
     static_assert(GBN == 16 || GBN % 32 == 0, "a key group scores 16 keys or whole groups of 32");
     constexpr bool K16 = GBN == 16;
@@ -579,13 +579,13 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
         }
     }
 
-    constexpr float kLazy = 8.f;
-    const float lazy_raw = kLazy / scale_log2e;   // the same margin in raw-score units
+    constexpr float kGuard = 4096.f;   // a lane's share of a tile's row sum at which the reference point is renewed
     float16_t o[2][2];      // [query block][32-dim block]
-    float m_run[2], l_run[2];   // running maximum of the query; the lane's share of its row sum
+    float m_run[2], mc_run[2], l_run[2];   // reference point of the query's exponentials (raw, and times scale * log2 e); the lane's share of its row sum
 #pragma unroll
     for (int b = 0; b < 2; b++) {
         m_run[b] = -INFINITY;
+        mc_run[b] = -INFINITY;
         l_run[b] = 0.f;
 #pragma unroll
         for (int d = 0; d < 2; d++)
@@ -748,40 +748,49 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
                         for (int r = 0; r < 16; r++)
                             if (32 * c + 8 * (r >> 2) + (r & 3) > rel) sc[b][c][r] = -INFINITY;
                 }
-                float mx = max3_raw(sc[b][0][0], sc[b][0][1], sc[b][0][2]);
-                mx = max_raw(mx, sc[b][0][3]);
+                // The reference point m of the exponentials (P = 2^((s - m) c)) is not tracked per tile: the block's P
+                // is computed against the current one, and the lane's share of the row sum -- needed anyway -- tells
+                // whether that was safe.  P >= 0, so a share below kGuard bounds every P of the lane below kGuard:
+                // nothing overflowed fp16, whose relative precision is the same everywhere below that, and O / l
+                // does not depend on m.  Only when some lane's share reaches kGuard (the first tile, where m is
+                // -inf and P comes out inf or NaN; later a score more than 12 binary orders above m) the true
+                // maximum of the block is taken, m raised to it, the accumulators rescaled and P computed again.
+                // On random data that happens once or twice per query block and sequence, so the 16 maximum
+                // instructions, the cross-lane exchange and the compare of the per-tile tracking are gone from
+                // the loop (they were a sixth of its vector instructions).
+                half8_t pb[4];
+                auto exp_block = [&](const float mc) {
+                    float lsum = 0.f;
 #pragma unroll
-                for (int i = 2; i < 16; i++) mx = max3_raw(mx, sc[b][i >> 3][(2 * i) & 15], sc[b][i >> 3][(2 * i + 1) & 15]);
-                mx = max_xor32(mx);   // the two lanes that share the query
-                // The reference point of the exponentials is a running maximum that is only raised when some
-                // query of the block exceeds it by more than kLazy binary orders of magnitude: P then lies in
-                // (0, 2^kLazy] instead of (0, 1], which fp16 holds with the same relative precision, the
-                // quotient O / l does not depend on the reference point, and the rescaling of the block's
-                // 34 accumulator registers runs for a few tiles per sequence instead of for most of them
-                // (a block of 32 queries of random data sees a new maximum in ~60 % of 128 tiles).
-                if (__builtin_amdgcn_ballot_w64(mx > m_run[b] + lazy_raw) != 0) {
+                    for (int g = 0; g < 4; g++) {
+                        uint32_t pw[4];
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {   // P rounded to fp16 (nearest even), as P.to(fp16)
+                            const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[b][g >> 1][8 * (g & 1) + 2 * i], scale_log2e, -mc));
+                            const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[b][g >> 1][8 * (g & 1) + 2 * i + 1], scale_log2e, -mc));
+                            pw[i] = as_u32(__builtin_convertvector(float2v_t{e0, e1}, half2_t));
+                            lsum = dot2(pw[i], 0x3c003c00u, lsum);   // the row sum takes the rounded values that multiply V
+                        }
+                        pb[g] = __builtin_bit_cast(half8_t, u32x4{pw[0], pw[1], pw[2], pw[3]});
+                    }
+                    return lsum;
+                };
+                float lsum = exp_block(mc_run[b]);
+                if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lsum < kGuard)) != 0, 0)) {   // wave-uniform, rare
+                    float mx = max3_raw(sc[b][0][0], sc[b][0][1], sc[b][0][2]);
+                    mx = max_raw(mx, sc[b][0][3]);
+#pragma unroll
+                    for (int i = 2; i < 16; i++) mx = max3_raw(mx, sc[b][i >> 3][(2 * i) & 15], sc[b][i >> 3][(2 * i + 1) & 15]);
+                    mx = max_xor32(mx);   // the two lanes that share the query
                     const float m_old = m_run[b];
                     const float m_new = max_raw(m_old, mx);
                     const float alpha = __builtin_amdgcn_exp2f((m_old - m_new) * scale_log2e);
                     m_run[b] = m_new;
+                    mc_run[b] = m_new * scale_log2e;
                     l_run[b] *= alpha;
 #pragma unroll
                     for (int d = 0; d < 2; d++) o[b][d] *= alpha;
-                }
-                const float mc = m_run[b] * scale_log2e;
-                half8_t pb[4];
-                float lsum = 0.f;
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    uint32_t pw[4];
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {   // P rounded to fp16 (nearest even), as P.to(fp16)
-                        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[b][g >> 1][8 * (g & 1) + 2 * i], scale_log2e, -mc));
-                        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[b][g >> 1][8 * (g & 1) + 2 * i + 1], scale_log2e, -mc));
-                        pw[i] = as_u32(__builtin_convertvector(float2v_t{e0, e1}, half2_t));
-                        lsum = dot2(pw[i], 0x3c003c00u, lsum);   // the row sum takes the rounded values that multiply V
-                    }
-                    pb[g] = __builtin_bit_cast(half8_t, u32x4{pw[0], pw[1], pw[2], pw[3]});
+                    lsum = exp_block(mc_run[b]);
                 }
                 l_run[b] += lsum;
                 // ---- O^T += V^T P^T

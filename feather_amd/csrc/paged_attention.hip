@@ -83,6 +83,7 @@ __device__ __forceinline__ void v_pairs(uint32_t wa, uint32_t wb, uint32_t out[4
 // workgroup whose split holds the new token's position ("owner") does the same for that token's K and V row of
 // its KV head, appends them to the cache and scores the token from LDS after the cached ones (wave 0, one extra
 // one-token step), so the cached tokens are read from memory and the new one never is.
+constexpr int kEarly = 2;             // FUSED: steps of a wave whose rows are requested before the query is ready
 constexpr int kFusedMaxPairs = 96;   // (group + 2) * n_part the LDS staging of the FUSED prologue holds
 
 template <int D, int MODE, bool FAST, bool FUSED = false>
@@ -405,6 +406,11 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         const float4_t *csp = reinterpret_cast<const float4_t *>(cs + ((int64_t)seq * (D / 2) + 4 * my_tt) * 2);
         cs01 = csp[0];                                             // (cos, sin) of elements 4 tt .. 4 tt + 3
         cs23 = csp[1];
+        // the wave's first step goes out behind the partial sums (memory returns in order: parking the sums waits for
+        // them, not for the rows), so the cache rows start to stream one round trip earlier than the query allows
+#pragma unroll
+        for (int f = 0; f < kEarly; f++)   // (a wave without such a step reads the split's first block: no branch, so the wait below counts loads)
+            load_step(steps[f], t_begin + kStepTok * (wave + kPaWaves * f));
 #pragma unroll
         for (int it = 0; it < kUnitsPerThread; it++) {
             const int u = threadIdx.x + it * kPaThreads;
@@ -414,10 +420,9 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
             }
         }
     }
-    // Phase B runs inside the first turn of the main loop, behind the loads of the wave's first steps: the cached
-    // K / V rows are in flight while the query is rotated and packed.  (The partial sums are parked in LDS before
-    // those loads go out: issued the other way round, the 64 destination registers of the rows would be live
-    // together with the partial sums' and one workgroup less would fit a CU.)
+    // Phase B runs behind the loads of the wave's first step.  (Only that step: with the rows of all four steps
+    // requested before the partial sums are parked, their 64 destination registers are live together with the
+    // partial sums' and one workgroup less fits a CU.)
     auto fused_phase_b = [&]() {
         constexpr int T8 = D / 8;
         const int slots = group + (owner ? 2 : 0);
@@ -462,23 +467,33 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
         }
     };
 
-    // The wave's steps are wave, wave + 4, ...; NF of them are in flight together: a wave has only
-    // a handful of steps, so their chains must overlap each other.  (FUSED: every wave makes the first turn,
-    // also one without steps, because that turn holds the workgroup barriers of the query's phase B.)
-    for (int st = wave; st < n_steps || (FUSED && st == wave); st += kPaWaves * NF) {
-        if (st != wave) {
+    // Phase B: the query is rotated and packed while the rows of the wave's first step are in flight (every wave
+    // takes part: the phase holds workgroup barriers).
+    if constexpr (FUSED) fused_phase_b();
+
+    // The wave's steps are wave, wave + 4, ...; NF of them are in flight together: a wave has only a handful of
+    // steps, so their chains must overlap each other.  The loads of a turn go out kAhead steps ahead of the
+    // arithmetic instead of all up front: when every workgroup of the grid asks for its rows at once the memory
+    // system is the bottleneck and a wave sits in the issue of its loads until there is room for them, so the
+    // arithmetic of the early steps fits under the stream of the later ones.
+    constexpr int kAhead = NF < 3 ? NF : 3;
+    for (int st = wave; st < n_steps; st += kPaWaves * NF) {
+        const bool first_turn = st == wave;
+        if (!first_turn) {
 #pragma unroll
             for (int f = 0; f < NF; f++)
                 if (st + kPaWaves * f < n_steps) fetch_ids(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
         }
 #pragma unroll
-        for (int f = 0; f < NF; f++)
-            if (st + kPaWaves * f < n_steps) load_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
-        if constexpr (FUSED)
-            if (st == wave) fused_phase_b();
+        for (int f = 0; f < kAhead; f++)
+            if (st + kPaWaves * f < n_steps && !(FUSED && first_turn && f < kEarly))
+                load_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
 #pragma unroll
-        for (int f = 0; f < NF; f++)
+        for (int f = 0; f < NF; f++) {
+            if (f + kAhead < NF && st + kPaWaves * (f + kAhead) < n_steps && !(FUSED && first_turn && f + kAhead < kEarly))
+                load_step(steps[f + kAhead], t_begin + kStepTok * (st + kPaWaves * (f + kAhead)));
             if (st + kPaWaves * f < n_steps) compute_step(steps[f], t_begin + kStepTok * (st + kPaWaves * f));
+        }
     }
 
     if constexpr (FUSED) {

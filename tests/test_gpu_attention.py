@@ -142,6 +142,34 @@ def test_flash_attention_rising_scores(dev, orc, mode, d, ramp):
     assert _nerr(got, want64) <= TOL
 
 
+@pytest.mark.parametrize("mode,d", [("E5M2", 64), ("E4M3", 64), ("E4M3", 256)])
+def test_flash_attention_denominator_of_rounded_p(dev, orc, mode, d):
+    """The one deliberate deviation from the reference's arithmetic, bounded by itself: the kernels divide by the
+    sum of the fp16-rounded P (the values that multiply V), the reference by the sum of P before rounding
+    (feather/routines/attention.py:80-82 against :90).  Both quotients are formed here in float64 from the decoded
+    operands: they differ by at most 2^-11 of the output scale (the rounding errors of a row's weights mostly
+    cancel: measured ~1e-5); the kernel -- whose exponentials refer to another point than the row maximum, so its
+    P round differently -- agrees with both to half the stated tolerance or better."""
+    from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
+    rng = np.random.default_rng(7 + d)
+    heads, L = 2, 512
+    q, k, v = _qkv(rng, heads, L, d, mode, orc)
+    out = flash_attention_fp8_acc_fp32_gpu(_dev_words(q, dev), _dev_words(k, dev), _dev_words(v, dev), L, d // 4,
+                                           mode=mode)
+    got = out.cpu().numpy().reshape(heads, L, d).astype(np.float64)
+    Q, K, V = (orc.decode_np(a, mode).reshape(heads, L, d) for a in (q, k, v))
+    S = np.einsum("hqd,hkd->hqk", Q, K) / np.sqrt(d)
+    P = np.exp(S - S.max(axis=-1, keepdims=True))
+    P16 = P.astype(np.float16).astype(np.float64)
+    num = np.einsum("hqk,hkd->hqd", P16, V)
+    ref_variant = num / P.sum(axis=-1, keepdims=True)        # the reference: l sums P before rounding
+    own_variant = num / P16.sum(axis=-1, keepdims=True)      # the kernels: l sums the rounded P
+    scale = np.abs(ref_variant).max()
+    assert np.abs(own_variant - ref_variant).max() / scale <= 2.0 ** -11
+    assert np.abs(got - own_variant).max() / scale <= 5e-4
+    assert np.abs(got - ref_variant).max() / scale <= TOL
+
+
 @pytest.mark.parametrize("d", [64, 128, 256])
 def test_flash_attention_e4m3_kernel_decode_codes(dev, orc, d):
     """E4M3 operands are decoded as the reference kernel does (gemv.py:83-88), not as OCP FP8: a zero-exponent

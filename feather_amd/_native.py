@@ -16,6 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libfeather_hip.so")
 
 OK, EINVAL, EMODE, ESHAPE, ELAUNCH = 0, -1, -2, -3, -4
+ABI_VERSION = 10300   # FEATHER_HIP_VERSION of the include/feather_hip.h these signatures were written against
 E5M2, E4M3 = 0, 1
 ROUND_RNE, ROUND_TRUNC = 0, 1
 SEM_KERNEL, SEM_IEEE = 0, 1
@@ -51,6 +52,7 @@ SIGNATURES = {
     "feather_paged_attn_fp8_static": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
                                              _i64, _i64, _i32, _f32, _vp]),
     "feather_decode_step_scratch_bytes": (_i64, [_vp, _i64, _i64]),
+    "feather_decode_step_attention_path": (_i32, [_vp, _i64, _i64]),
     "feather_decode_step": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp]),
     "feather_add_rmsnorm_pack": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _vp]),
     "feather_rope_append": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
@@ -92,6 +94,11 @@ def lib() -> ctypes.CDLL:
                     fn = getattr(L, name)  # AttributeError here = header and library out of step
                     fn.restype = res
                     fn.argtypes = args
+                got = L.feather_version()
+                if got // 100 != ABI_VERSION // 100:   # major.minor: any signature or struct change
+                    raise RuntimeError(
+                        f"{LIB_PATH} reports version {got}, this binding was written against {ABI_VERSION}: "
+                        "rebuild the library with `python -m feather_amd.build`")
                 _lib = L
     return _lib
 

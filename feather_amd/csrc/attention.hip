@@ -903,6 +903,8 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
         return ((rows + queries_per_group - 1) / queries_per_group * seqs * a.n_heads + 255) / 256;
     };
     switch (d) {
+        case 32:   // narrower than anything the reference's tl.dot accepts (d / 4 >= 16); one MFMA k-step per score
+            return launch_attn<32, MODE, 4, 4, 64, 2, VC>(a, s);
         case 64:   // all four query blocks of a wave share every K fragment
             // eight waves halve the staging work per query (-2 % time); a causal tile of 512 queries
             // would idle its early waves through too many masked key tiles
@@ -931,7 +933,7 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
             return launch_attn<512, MODE, 1, 1, 32, 1, VC>(a, s);
         }
     }
-    set_error("feather_flash_attn_fp8: head dim %lld not supported (64, 128, 256, 512)", (long long)d);
+    set_error("feather_flash_attn_fp8: head dim %lld not supported (32, 64, 128, 256, 512)", (long long)d);
     return FEATHER_ESHAPE;
 }
 
@@ -978,8 +980,8 @@ extern "C" int feather_flash_attn_fp8_varlen(const void *q, const void *k, const
     FEATHER_CHECK(max_seqlen <= total_rows && total_rows < (1ll << 30), FEATHER_ESHAPE,
                   "%s: max_seqlen=%lld must not exceed total_rows=%lld (< 2^30)", me, (long long)max_seqlen,
                   (long long)total_rows);
-    FEATHER_CHECK(d == 64 || d == 128 || d == 256 || d == 512, FEATHER_ESHAPE,
-                  "%s: head dim %lld not supported (64, 128, 256, 512)", me, (long long)d);
+    FEATHER_CHECK(d == 32 || d == 64 || d == 128 || d == 256 || d == 512, FEATHER_ESHAPE,
+                  "%s: head dim %lld not supported (32, 64, 128, 256, 512)", me, (long long)d);
     if (n_heads == 0 || n_seq == 0 || max_seqlen == 0) return FEATHER_OK;
     FEATHER_CHECK(q && k && v && out_f32 && cu_seqlens, FEATHER_EINVAL, "%s: null pointer", me);
     FEATHER_CHECK(aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out_f32, 16) && aligned(cu_seqlens, 4),

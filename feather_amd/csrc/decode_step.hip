@@ -409,6 +409,18 @@ __global__ __launch_bounds__(kDsThreads) void step_prologue_kernel(
     }
 }
 
+// Per-sequence status of a step whose layers do not write it (the generic path writes it from the first layer's
+// rotary kernel; a model without layers has none): the same rule as rope_append_kernel.
+__global__ void seq_status_kernel(const int32_t *__restrict__ ctx_lens, const int32_t *__restrict__ block_tables, int batch,
+                                  int block_size, int max_blocks, int n_blocks, int pos_limit, int32_t *__restrict__ status) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= batch) return;
+    const int pos_raw = ctx_lens[b];
+    const bool pos_ok = pos_raw >= 0 && pos_raw < pos_limit;
+    const int blk = block_tables[(int64_t)b * max_blocks + (pos_ok ? pos_raw : 0) / block_size];
+    status[b] = pos_ok ? ((unsigned)blk < (unsigned)n_blocks ? 0 : 2) : 1;
+}
+
 // K slices per GEMV: enough 64-row tiles x slices to cover the 256 CUs, at most one slice per
 // 256-column chunk (the launcher's own clamp, repeated here to size the partial buffers)
 static int plan_splits(int64_t M, int64_t K) {
@@ -503,6 +515,9 @@ static int run_step(const feather_decoder_t *dec, const int32_t *tokens, const i
                            dec->max_blocks, dec->n_blocks, max_ctx, n_splits, log2_theta, cs, plan, ctx_after, status);
     } else {
         hipLaunchKernelGGL(embed_kernel, dim3(batch), dim3(kDsThreads), 0, s, (const _Float16 *)dec->embed_f16, tokens, h, H);
+        if (dec->n_layers == 0 && status)     // no rotary kernel will write it
+            hipLaunchKernelGGL(seq_status_kernel, dim3(1), dim3(64), 0, s, ctx_lens, block_tables, batch, dec->block_size,
+                               dec->max_blocks, dec->n_blocks, max_ctx, status);
     }
     DS_CHECK(check_launch("feather_decode_step (embed)"));
     const float *pending = nullptr;                       // output of the previous down projection, not yet added
@@ -583,6 +598,11 @@ static int check_decoder(const feather_decoder_t *dec, int64_t batch, int64_t ma
     return FEATHER_OK;
 }
 
+extern "C" int feather_decode_step_attention_path(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx) {
+    if (check_decoder(dec, batch, max_ctx, "feather_decode_step_attention_path") != FEATHER_OK) return -1;
+    return plan_step(dec, batch, max_ctx).fused_attn ? 1 : 0;
+}
+
 extern "C" int64_t feather_decode_step_scratch_bytes(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx) {
     if (check_decoder(dec, batch, max_ctx, "feather_decode_step_scratch_bytes") != FEATHER_OK) return -1;
     return step_scratch_bytes(dec, batch, max_ctx);
@@ -651,6 +671,9 @@ extern "C" int feather_rope_append(const void *qkv_f32, int64_t n_part, int64_t 
                       n_blocks > 0 && n_blocks < (1ll << 31) && max_blocks * block_size < (1ll << 31),
                   FEATHER_EINVAL, "%s: bad shape", me);
     FEATHER_CHECK(d > 0 && d % 8 == 0 && d <= 1024, FEATHER_ESHAPE, "%s: head dim %lld is not a multiple of 8", me, (long long)d);
+    FEATHER_CHECK(n_q_heads < (1ll << 31) && n_kv_heads < (1ll << 31) && (n_q_heads + 2 * n_kv_heads) * (d / 8) <= 65535ll * kRopeThreads, FEATHER_ESHAPE,
+                  "%s: (n_q_heads + 2 n_kv_heads) * d / 8 = %lld exceeds the grid (%lld)", me,
+                  (long long)((n_q_heads + 2 * n_kv_heads) * (d / 8)), 65535ll * kRopeThreads);
     FEATHER_CHECK(n_part >= 1 && n_part <= 64 && part_stride >= 0 && part_stride % 4 == 0, FEATHER_EINVAL,
                   "%s: n_part must be in [1, 64] and part_stride a non-negative multiple of 4", me);
     FEATHER_CHECK(rope_theta > 0.f, FEATHER_EINVAL, "%s: rope_theta must be positive", me);

@@ -265,7 +265,7 @@ static int64_t launch_copy128(const void *src, void *dst, int64_t n16, hipStream
 
 using namespace feather;
 
-extern "C" int feather_version(void) { return 100; }
+extern "C" int feather_version(void) { return FEATHER_HIP_VERSION; }
 
 extern "C" const char *feather_last_error(void) { return g_err; }
 

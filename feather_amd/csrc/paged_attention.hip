@@ -760,11 +760,13 @@ int paged_attn_launch(const void *q, const void *k_cache, const void *v_cache, c
     if (mode == FEATHER_E5M2) {
         if (d == 64) FEATHER_PA(64, FEATHER_E5M2);
         if (d == 128) FEATHER_PA(128, FEATHER_E5M2);
-        FEATHER_PA(256, FEATHER_E5M2);
+        if (d == 256) FEATHER_PA(256, FEATHER_E5M2);
+        FEATHER_PA(512, FEATHER_E5M2);
     }
     if (d == 64) FEATHER_PA(64, FEATHER_E4M3);
     if (d == 128) FEATHER_PA(128, FEATHER_E4M3);
-    FEATHER_PA(256, FEATHER_E4M3);
+    if (d == 256) FEATHER_PA(256, FEATHER_E4M3);
+    FEATHER_PA(512, FEATHER_E4M3);
 #undef FEATHER_PA
 }
 
@@ -793,8 +795,8 @@ extern "C" int feather_paged_attn_fp8(const void *q, const void *k_cache, const 
     FEATHER_CHECK(n_q_heads % n_kv_heads == 0, FEATHER_ESHAPE, "%s: n_q_heads=%lld not a multiple of n_kv_heads=%lld",
                   me, (long long)n_q_heads, (long long)n_kv_heads);
     FEATHER_CHECK(n_q_heads / n_kv_heads <= 16, FEATHER_ESHAPE, "%s: at most 16 query heads per KV head", me);
-    FEATHER_CHECK(d == 64 || d == 128 || d == 256, FEATHER_ESHAPE, "%s: head dim %lld not supported (64, 128, 256)", me,
-                  (long long)d);
+    FEATHER_CHECK(d == 64 || d == 128 || d == 256 || d == 512, FEATHER_ESHAPE,
+                  "%s: head dim %lld not supported (64, 128, 256, 512)", me, (long long)d);
     FEATHER_CHECK(max_ctx <= max_blocks * block_size, FEATHER_ESHAPE, "%s: max_ctx exceeds the block table", me);
     FEATHER_CHECK(scale > 0.f, FEATHER_EINVAL, "%s: scale must be positive (the running maximum is kept on raw scores)", me);
     if (n_seq == 0) return FEATHER_OK;

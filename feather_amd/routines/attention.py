@@ -41,8 +41,8 @@ def flash_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: torch.
     if seq_len < 0 or h_dim <= 0:
         raise ValueError(f"bad shape: seq_len={seq_len}, h_dim={h_dim}")
     d = 4 * h_dim
-    if d not in (64, 128, 256, 512):
-        raise ValueError(f"head dim {d} (h_dim={h_dim} words) not supported: 64, 128, 256 or 512")
+    if d not in (32, 64, 128, 256, 512):
+        raise ValueError(f"head dim {d} (h_dim={h_dim} words) not supported: 32, 64, 128, 256 or 512")
     q, k, v = N.as_words(q, "q"), N.as_words(k, "k"), N.as_words(v, "v")
     per_head = seq_len * h_dim
     if per_head == 0 or q.numel() % per_head != 0:
@@ -107,8 +107,8 @@ def flash_attention_fp8_varlen_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v:
     n_heads, total, dw = q.shape
     n_kv = k.shape[0]
     d = 4 * dw
-    if d not in (64, 128, 256, 512):
-        raise ValueError(f"head dim {d} not supported: 64, 128, 256 or 512")
+    if d not in (32, 64, 128, 256, 512):
+        raise ValueError(f"head dim {d} not supported: 32, 64, 128, 256 or 512")
     if n_kv == 0 or n_heads % n_kv != 0:
         raise ValueError(f"n_heads={n_heads} is not a multiple of n_kv_heads={n_kv}")
     if cu_seqlens.dtype != torch.int32 or cu_seqlens.dim() != 1 or cu_seqlens.numel() < 1 or not cu_seqlens.is_cuda:

@@ -99,6 +99,16 @@ class PackedDecoder:
             n += 4 * (lay["w_qkv"].numel() + lay["w_o"].numel() + lay["w_gate_up"].numel() + lay["w_down"].numel())
         return n
 
+    def attention_path(self, batch: int, max_ctx: int | None = None) -> str:
+        """Which attention path a step of this shape takes: ``"fused"`` (rotary embedding, query packing and the
+        K/V append inside the attention kernel; the new token is scored after the cached ones) or ``"generic"``
+        (separate rotary / append kernel, then paged attention in position order)."""
+        max_ctx = self.max_blocks * self.cfg.block_size if max_ctx is None else int(max_ctx)
+        r = int(N.lib().feather_decode_step_attention_path(ctypes.byref(self._c), int(batch), max_ctx))
+        if r < 0:
+            raise ValueError(N.lib().feather_last_error().decode())
+        return "fused" if r == 1 else "generic"
+
     def step(self, token_ids: torch.Tensor, block_tables: torch.Tensor, ctx_lens: torch.Tensor,
              max_ctx: int | None = None, out: torch.Tensor | None = None,
              status: torch.Tensor | None = None) -> torch.Tensor:

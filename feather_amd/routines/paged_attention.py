@@ -39,8 +39,8 @@ def paged_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k_cache: torch.Tensor, v_c
     if dw != dw2:
         raise ValueError(f"head dim mismatch: q has {dw} words per head, cache has {dw2}")
     d = 4 * dw
-    if d not in (64, 128, 256):
-        raise ValueError(f"head dim {d} not supported: 64, 128 or 256")
+    if d not in (64, 128, 256, 512):
+        raise ValueError(f"head dim {d} not supported: 64, 128, 256 or 512")
     if n_q_heads % n_kv_heads != 0 or n_q_heads // n_kv_heads > 16:
         raise ValueError(f"n_q_heads={n_q_heads} must be a multiple of n_kv_heads={n_kv_heads} with ratio <= 16")
     if block_tables.dtype != torch.int32 or context_lens.dtype != torch.int32:

@@ -52,7 +52,10 @@ extern "C" {
 #define FEATHER_TAIL_REFERENCE 1  /* keys past seq_len in the last 64-key tile count as zero rows
                                      (attention.py:57-59) */
 
-/* Library version (major * 10000 + minor * 100 + patch). */
+/* Library version (major * 10000 + minor * 100 + patch); FEATHER_HIP_VERSION is the version of this header.
+ * A change of any signature or struct below raises the minor number: a binding must refuse a library whose
+ * feather_version() differs from the header it was written against in major or minor. */
+#define FEATHER_HIP_VERSION 10300
 int feather_version(void);
 
 /* Message for the last non-zero return code on this thread ("" if none). */
@@ -134,7 +137,8 @@ int feather_dot_fp16(const void *x1, const void *x2, void *out_f32, void *scratc
 /* Non-causal attention forward on packed Q/K/V of fixed length: for each of n_heads
  * independent heads, out[h] = softmax(Q K^T * scale) V, Q/K/V [L, d/4] words,
  * out [L, d] fp32; scores fp32, P rounded to fp16 before P.V, fp32 output.
- * d in {64, 128, 256, 512}.  kv_group > 1 maps query head h to K/V head
+ * d in {32, 64, 128, 256, 512}; any other head dim returns FEATHER_ESHAPE (the reference kernel takes
+ * power-of-two d >= 64, attention.py:28-41, :145: its tl.dot needs d / 4 >= 16).  kv_group > 1 maps query head h to K/V head
  * h / kv_group (K/V then hold n_heads / kv_group heads).  scale must be positive.
  * Replaces flash_attention_fp8_e5m2_acc_fp32_gpu
  * (feather/routines/attention.py:110-179) at n_heads = 1, mode = E5M2,
@@ -185,6 +189,7 @@ int64_t feather_paged_attn_scratch_bytes(int64_t n_seq, int64_t n_q_heads, int64
  *   out_f32      [n_seq, n_q_heads, d] fp32, and / or
  *   out_packed   [n_seq, n_q_heads * d / 4] words: the same result rounded fp32 -> fp16 -> FP8 of `mode`
  *                (as feather_quant_pack_f32), the packed operand of a following GEMV; either may be NULL
+ * d in {64, 128, 256, 512} (any other head dim returns FEATHER_ESHAPE); at most 16 query heads per KV head.
  * Query head h uses KV head h / (n_q_heads / n_kv_heads).  Table entries of positions below
  * ctx_lens[s] must be blocks of the cache; an entry outside [0, n_blocks) is read as the last block
  * (a wrong result for that sequence, never an access outside the cache).  Entries past the context
@@ -202,7 +207,10 @@ int feather_paged_attn_fp8(const void *q, const void *k_cache, const void *v_cac
  * feather_paged_attn_scratch_bytes() exceeds that size is rejected with FEATHER_ESHAPE.  The call
  * allocates and frees nothing.  All calls on one GPU share the buffer: calls that overlap on one
  * GPU (different streams, or threads) race; calls on one stream are ordered and safe.  Nothing in
- * the buffer needs clearing between calls.  Results are bit-identical to feather_paged_attn_fp8. */
+ * the buffer needs clearing between calls.  Results are bit-identical to feather_paged_attn_fp8.
+ * The first call on a device looks up the buffer's device address (hipGetSymbolAddress: no allocation, no stream
+ * work, but it may load the code object): make that call before a stream capture begins; later calls only
+ * enqueue kernels and can be captured. */
 #define FEATHER_PAGED_ATTN_STATIC_SCRATCH_BYTES (4 << 20)
 int feather_paged_attn_fp8_static(const void *q, const void *k_cache, const void *v_cache, const void *block_tables,
                                   const void *ctx_lens, void *out_f32, void *out_packed, int64_t n_seq,
@@ -246,6 +254,13 @@ typedef struct feather_decoder {
 
 /* Bytes of scratch feather_decode_step needs (256-byte aligned buffer); -1 for a bad configuration. */
 int64_t feather_decode_step_scratch_bytes(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx);
+
+/* Which attention path feather_decode_step takes for this configuration: 1 = the attention kernel with the
+ * rotary embedding, query packing and K/V append in its prologue (head_dim 64, power-of-two block_size >= 4,
+ * batch <= 64: the new token is scored from registers after the cached ones), 0 = separate rotary / append kernel
+ * followed by feather_paged_attn_fp8 (the new token is read back from the cache in position order), -1 = bad
+ * configuration.  The two differ in the order of the softmax's additions only.  No reference counterpart. */
+int feather_decode_step_attention_path(const feather_decoder_t *dec, int64_t batch, int64_t max_ctx);
 
 /* token_ids [batch] int32, block_tables [batch, max_blocks] int32, ctx_lens [batch] int32 (tokens
  * already in the cache; the caller adds 1 after the step), logits [batch, vocab] fp32.

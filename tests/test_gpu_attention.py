@@ -44,6 +44,8 @@ def _qkv(rng, heads, L, d, mode, orc, ints=False):
     ("E4M3", 1, 300, 256), ("E4M3", 1, 7, 256),
     # the same split at d = 512 (32-key tiles, 16 keys per group on the 16x16x16 MFMA)
     ("E4M3", 2, 100, 512), ("E5M2", 1, 200, 512), ("E4M3", 1, 50, 512), ("E5M2", 2, 81, 512), ("E4M3", 1, 3, 512),
+    # d = 32: narrower than the reference's tl.dot takes; one MFMA k-step per score, half a tile of staging threads
+    ("E5M2", 3, 300, 32), ("E4M3", 2, 257, 32), ("E5M2", 1, 64, 32), ("E4M3", 1, 5, 32), ("E5M2", 8, 1024, 32),
 ])
 def test_flash_attention_vs_oracle(dev, orc, mode, heads, L, d):
     from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
@@ -75,7 +77,7 @@ def test_flash_attention_reference_signature_and_ints(dev, orc):
     assert np.abs(out.cpu().numpy() - sd.numpy()).max() <= 2e-3
 
 
-@pytest.mark.parametrize("L,d", [(1, 64), (5, 64), (63, 64), (65, 64), (70, 64), (130, 64),
+@pytest.mark.parametrize("L,d", [(1, 32), (65, 32), (1, 64), (5, 64), (63, 64), (65, 64), (70, 64), (130, 64),
                                  (70, 256), (100, 256), (40, 512), (81, 512)])   # wide heads: two key groups per tile
 def test_flash_attention_ragged_tails(dev, orc, L, d):
     from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
@@ -334,6 +336,8 @@ def test_varlen_attention_random_shapes(dev, orc, seed):
 @pytest.mark.parametrize("mode,n_seq,Hq,Hkv,d,bs,max_ctx", [
     ("E5M2", 3, 8, 2, 64, 16, 100), ("E4M3", 4, 32, 4, 64, 16, 700), ("E4M3", 2, 4, 4, 128, 16, 300),
     ("E5M2", 2, 16, 1, 64, 8, 90), ("E4M3", 1, 2, 1, 256, 32, 257),
+    # d = 512 (one step in flight per wave, 96 KB of LDS for the wave merge): one split, three splits, odd block size
+    ("E4M3", 2, 4, 2, 512, 16, 200), ("E5M2", 3, 8, 1, 512, 16, 1300), ("E4M3", 2, 2, 2, 512, 12, 100),
 ])
 def test_paged_attention_vs_oracle(dev, orc, mode, n_seq, Hq, Hkv, d, bs, max_ctx):
     from feather_amd.routines.paged_attention import paged_attention_fp8_acc_fp32_gpu
@@ -463,6 +467,7 @@ def test_paged_attention_config_shape(dev, orc):
     ("E5M2", 16, 8, 64, [513, 100, 512, 0] * 4, False),
     ("E4M3", 2, 1, 256, [130, 64, 0, 257], False),           # d = 256 with the key tiles split between wave groups
     ("E4M3", 16, 8, 256, [257, 100] * 8, True),              # d = 256, 32 queries per wave (>= 256 workgroups)
+    ("E5M2", 4, 2, 32, [70, 0, 300, 1], True), ("E4M3", 2, 1, 32, [129, 64], False),     # d = 32
 ])
 def test_varlen_attention_vs_oracle(dev, orc, mode, n_heads, n_kv, d, lens, causal):
     from feather_amd.routines.attention import flash_attention_fp8_varlen_acc_fp32_gpu

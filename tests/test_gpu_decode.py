@@ -42,21 +42,25 @@ def _assert_untouched_elsewhere(got: np.ndarray, before: np.ndarray, bt, ctx, bs
     assert np.array_equal(got[mask], before[mask]), f"{what}: a cache row outside the appended slots changed"
 
 
-@pytest.mark.parametrize("mode,hidden,nq,nkv,inter,block", [
-    ("E4M3", 512, 8, 2, 1024, 16), ("E5M2", 256, 4, 4, 512, 16), ("E4M3", 1024, 16, 1, 1536, 16), ("E4M3", 320, 5, 1, 704, 16),
+@pytest.mark.parametrize("mode,hidden,nq,nkv,inter,block,hd,path", [
+    ("E4M3", 512, 8, 2, 1024, 16, 64, "fused"), ("E5M2", 256, 4, 4, 512, 16, 64, "fused"),
+    ("E4M3", 1024, 16, 1, 1536, 16, 64, "fused"), ("E4M3", 320, 5, 1, 704, 16, 64, "fused"),
     # a block size that is not a power of two: the step runs the stand-alone rotary kernel and the generic attention
-    ("E4M3", 512, 8, 2, 1024, 12), ("E5M2", 256, 4, 2, 512, 8)])
-def test_decode_step_vs_oracle(orc, mode, hidden, nq, nkv, inter, block):
+    ("E4M3", 512, 8, 2, 1024, 12, 64, "generic"), ("E5M2", 256, 4, 2, 512, 8, 64, "fused"),
+    # wider heads take the generic path whatever the block size
+    ("E4M3", 512, 4, 2, 1024, 16, 128, "generic"), ("E5M2", 512, 2, 1, 768, 16, 256, "generic")])
+def test_decode_step_vs_oracle(orc, mode, hidden, nq, nkv, inter, block, hd, path):
     from feather_amd.routines.decode import DecoderConfig, PackedDecoder, random_weights
     from oracle import decode_ref
     dev = torch.device("cuda:0")
-    cfg = DecoderConfig(n_layers=2, hidden=hidden, n_q_heads=nq, n_kv_heads=nkv, head_dim=64, inter=inter, vocab=1000,
+    cfg = DecoderConfig(n_layers=2, hidden=hidden, n_q_heads=nq, n_kv_heads=nkv, head_dim=hd, inter=inter, vocab=1000,
                         block_size=block)
-    fused = block & (block - 1) == 0                           # the attention kernel with the fused rotary prologue
     B, max_blocks = 3, 6
     n_blocks = B * max_blocks + 2
     w = random_weights(cfg, seed=hidden)
     dec = PackedDecoder(cfg, w, n_blocks=n_blocks, max_blocks=max_blocks, mode=mode, device=dev)
+    assert dec.attention_path(B) == path                       # the library says which path ran; the oracle follows it
+    fused = path == "fused"                                    # the attention kernel with the fused rotary prologue
     g = torch.Generator().manual_seed(1)
     bt = torch.randperm(n_blocks, generator=g)[: B * max_blocks].to(torch.int32).view(B, max_blocks)
     ctx = torch.tensor([5, 40, 0], dtype=torch.int32)
@@ -268,15 +272,19 @@ def test_decode_step_tinyllama_full_size(orc):
         feather.dot(dec.lm_head[:4096], dec.lm_head[:4096], mode=mode)      # eager work between the replays
 
 
-def test_decode_step_reports_full_cache_and_bad_block_ids():
+@pytest.mark.parametrize("hd,nq,nkv,n_layers,path", [(64, 4, 2, 2, "fused"), (128, 2, 1, 2, "generic"),
+                                                      (64, 4, 2, 0, "fused"), (128, 2, 1, 0, "generic")])
+def test_decode_step_reports_full_cache_and_bad_block_ids(hd, nq, nkv, n_layers, path):
     """A sequence whose block table is full, a negative length and a table entry outside the cache are
-    reported in `status` and write nothing; the other sequences of the batch are unaffected."""
+    reported in `status` and write nothing; the other sequences of the batch are unaffected.  Both attention
+    paths, and a model without layers (whose status no layer kernel writes)."""
     from feather_amd.routines.decode import DecoderConfig, PackedDecoder, random_weights
     dev = torch.device("cuda:0")
-    cfg = DecoderConfig(n_layers=2, hidden=256, n_q_heads=4, n_kv_heads=2, head_dim=64, inter=512, vocab=100)
+    cfg = DecoderConfig(n_layers=n_layers, hidden=256, n_q_heads=nq, n_kv_heads=nkv, head_dim=hd, inter=512, vocab=100)
     B, max_blocks, n_blocks = 4, 3, 12
     cap = max_blocks * cfg.block_size
     dec = PackedDecoder(cfg, random_weights(cfg), n_blocks=n_blocks, max_blocks=max_blocks, device=dev)
+    assert dec.attention_path(B) == path
     g = torch.Generator().manual_seed(0)
     for lay in dec.layers:
         for name in ("k_cache", "v_cache"):

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
 def test_version_and_error_string():
     from feather_amd import _native as N
     L = N.lib()
-    assert L.feather_version() >= 100
+    assert L.feather_version() // 100 == N.ABI_VERSION // 100      # header, library and binding agree (major.minor)
     assert isinstance(L.feather_last_error(), bytes)
     assert L.feather_dot_scratch_bytes() >= 64 + 4
     assert L.feather_paged_attn_scratch_bytes(32, 32, 64, 4096) == 32 * 32 * 8 * 66 * 4
@@ -86,6 +86,13 @@ def test_c_abi_argument_checks_without_gpu():
                                  10000.0, N.E4M3, None) == N.ESHAPE
     assert L.feather_rope_append(None, 1, 0, None, None, None, None, None, None, None, None, 2, 4, 2, 64, 16, 4, 0,
                                  10000.0, N.E4M3, None) == N.EINVAL                  # n_blocks = 0
+    assert L.feather_rope_append(None, 1, 0, None, None, None, None, None, None, None, None, 2, 1 << 20, 2, 1024, 16, 4, 8,
+                                 10000.0, N.E4M3, None) == N.ESHAPE                  # more (head, 8-element) items than the grid holds
+    assert b"exceeds the grid" in L.feather_last_error()
+    assert L.feather_flash_attn_fp8_varlen(None, None, None, None, None, 1, 8, 8, 1, 16, 1, N.E5M2, 0.1, 0, None) == N.ESHAPE
+    assert b"head dim 16" in L.feather_last_error()                                 # 32, 64, 128, 256, 512 only
+    assert L.feather_paged_attn_fp8(None, None, None, None, None, None, None, None, 1, 8, 4, 32, 16, 4, 8, 64, N.E5M2,
+                                    0.1, None) == N.ESHAPE                           # paged decode: 64, 128, 256, 512
     assert L.feather_paged_cache_write(None, None, 0, None, None, None, None, None, 1, 4, 2, 64, 16, 4, -1, N.E5M2,
                                        None) == N.EINVAL
 

@@ -74,3 +74,47 @@ def test_static_scratch_rejects_oversized_problem(dev):
                                          N.E4M3, 0.1, None)
     assert rc == N.ESHAPE
     assert b"built-in buffer" in L.feather_last_error()
+
+
+def test_static_entry_allocates_nothing_and_replays_in_a_graph(dev):
+    """Free device memory is the same before and after calls of the allocation-free entry point, and a captured
+    call replays to the bits of the eager call (the first call on a device, which looks up the buffer's address,
+    is made before the capture, as the header asks)."""
+    from feather_amd import _native as N
+    L = N.lib()
+    P = _problem(dev, 21, n_seq=8, Hq=16, Hkv=2, d=64, bs=16, max_ctx=1500, mode="E4M3")       # 3 splits + merge
+    want = _run(P, True, dev)                                   # first use on the device: outside any capture
+    out = torch.full((P["n_seq"], P["Hq"], P["d"]), float("nan"), dtype=torch.float32, device=dev)
+    code, scale = N.mode_code(P["mode"]), float(P["d"]) ** -0.5
+    n_blocks = P["kc"].numel() * 4 // (P["Hkv"] * P["bs"] * P["d"])
+    ptrs = [P[k].data_ptr() for k in ("q", "kc", "vc", "bt", "ctx")]
+
+    def call():
+        shape = (P["n_seq"], P["Hq"], P["Hkv"], P["d"], P["bs"], P["max_blocks"], n_blocks, P["max_ctx"], code, scale,
+                 N.stream_ptr(dev))
+        N.check(L.feather_paged_attn_fp8_static(*ptrs, out.data_ptr(), None, *shape))
+
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info(dev)
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info(dev)
+    assert free1 == free0, f"free device memory changed across the calls: {free0} -> {free1}"
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    other = _problem(dev, 22, n_seq=4, Hq=8, Hkv=2, d=64, bs=16, max_ctx=900, mode="E4M3")
+    for _ in range(3):
+        out.fill_(float("nan"))
+        _run(other, True, dev)                                  # eager work on the same buffer between the replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))

@@ -7,10 +7,14 @@ A "step" is one E4M3-packed GEMV of the 16384 x 16384 workload (FP32 accumulate)
 operands already resident in HBM.  Four distinct packed matrices (1 GiB in total) are
 rotated so that neither L2 nor the 256 MB Infinity Cache can serve the stream.  The single
 JSON line printed at the end carries the headline value (microseconds per GEMV), the
-roofline record of the GEMV kernel and the CPU baseline (torch-CPU restatement of the
-reference's decode + fp32 matvec, timed on the host cores of this box); `extra` holds the
-other workloads of the metric (E5M2 GEMV, 8192^2, dot, flash attention vs fp16 SDPA, paged
-decode).
+roofline record of the GEMV kernel -- with the matrix-core record of the metric's second half,
+flash attention d = 64 L = 8192, nested in it -- and the CPU baseline (torch-CPU restatement of
+the reference's pack + decode + fp32 compute, timed on the host cores of this box, one leg per
+configuration); `extra` holds the other workloads (the reference harness's GEMV grid in both
+modes, dot, pack / unpack, flash attention vs fp16 SDPA, paged decode, the decode step) with a
+roofline record each (`extra.roofline` HBM bound, `extra.roofline_mfma` matrix-core bound);
+every record says how it was timed ("events": back-to-back calls between HIP events; "graph":
+replay of captured calls, for kernels shorter than the host's per-call cost).
 """
 from __future__ import annotations
 
@@ -26,6 +30,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_F16_TFLOPS = 2500.0  # dense fp16/bf16, published
+MFMA_PEAK_F8_TFLOPS = 5000.0   # dense fp8/bf8, published
 WARM_MS = 40.0                  # warm-up time of the attention series (ours and SDPA alike)
 
 
@@ -84,6 +89,16 @@ def gpu_time_graph_us(fn, calls, sync, replays=10):
     return start.elapsed_time(stop) * 1000.0 / (replays * calls)
 
 
+def gpu_time_auto_us(fn, calls, steps, warmup, sync, warm_ms=0.0):
+    """(microseconds per call, timing method).  Back-to-back calls between HIP events ("events") unless a call
+    is shorter than the host's per-call cost (~12 us of wrapper and dispatch): then the device time alone, from
+    the replay of `calls` captured invocations ("graph").  One method per figure, never the smaller of two."""
+    us = gpu_time_us(fn, steps, warmup, sync, warm_ms)
+    if us >= 12.0:
+        return us, "events"
+    return gpu_time_graph_us(fn, calls, sync), "graph"
+
+
 def _source_hash(rel_paths) -> str:
     """sha256 (first 16 hex digits) over the kernel sources a counter figure belongs to."""
     import hashlib
@@ -114,17 +129,58 @@ def load_traffic() -> dict:
     return out
 
 
-def roofline_record(traffic_table, key, kernel, algorithmic_bytes, us, launches_per_call=1):
+def load_mfma_busy() -> dict:
+    """Matrix-core busy fraction per attention workload from the committed rocprofv3 counter summary: lines
+    `mfma_busy <key> <SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CYCLES per SIMD> <sha> <source>[,<source>...]`; stale figures
+    (kernel source changed since) are reported as null."""
+    out = {}
+    path = os.path.join(ROOT, "profiles", "bench_sq_counters.md")
+    if not os.path.exists(path):
+        return out
+    for ln in open(path):
+        f = ln.split()
+        if len(f) == 5 and f[0] == "mfma_busy":
+            try:
+                fresh = _source_hash(f[4].split(",")) == f[3]
+            except OSError:
+                fresh = False
+            out[f[1]] = (float(f[2]), fresh)
+    return out
+
+
+def roofline_record(traffic_table, key, kernel, algorithmic_bytes, us, launches_per_call=1, timing="events", note=None):
     """`roofline`-style record of an HBM-bound workload: achieved = algorithmic bytes / measured time."""
     achieved = algorithmic_bytes / (us * 1e-6) / 1e9
     t = traffic_table.get(key)
     rec = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": t[0] if t and t[1] else None, "kernel": kernel,
-           "algorithmic_bytes": int(algorithmic_bytes), "us": round(us, 3)}
+           "algorithmic_bytes": int(algorithmic_bytes), "us": round(us, 3), "timing": timing}
     if t and not t[1]:
         rec["traffic_note"] = "stale: the kernel source changed since the counters in profiles/bench_hbm_traffic.md were taken"
     if launches_per_call != 1:
         rec["launches_per_call"] = launches_per_call
+    if note:
+        rec["note"] = note
+    return rec
+
+
+def mfma_record(busy_table, key, kernel, flops, us, fp8_share, sdpa_us=None):
+    """`roofline`-style record of a matrix-core-bound workload.  `peak` is the dense fp16 MFMA peak; when a share of
+    the flops runs at the FP8 rate (the E5M2 score product on the bf8 matrix instructions) `peak_blended` is the rate
+    at which the same flop mix would run with every matrix instruction at its own peak, and both fractions are given."""
+    achieved = flops / (us * 1e-6) / 1e12
+    blended = 1.0 / (fp8_share / MFMA_PEAK_F8_TFLOPS + (1.0 - fp8_share) / MFMA_PEAK_F16_TFLOPS)
+    b = busy_table.get(key)
+    rec = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+           "frac": round(achieved / MFMA_PEAK_F16_TFLOPS, 4), "peak_blended": round(blended, 1),
+           "frac_blended": round(achieved / blended, 4), "fp8_rate_flop_share": fp8_share, "traffic": None,
+           "kernel": kernel, "flops": int(flops), "us": round(us, 1), "timing": "events",
+           "mfma_busy": b[0] if b and b[1] else None}
+    if b and not b[1]:
+        rec["mfma_busy_note"] = "stale: the kernel source changed since the counters in profiles/bench_sq_counters.md were taken"
+    if sdpa_us is not None:
+        rec["sdpa_fp16_same_gpu_us"] = round(sdpa_us, 1)
+        rec["speedup_vs_sdpa_fp16"] = round(sdpa_us / us, 3)
     return rec
 
 
@@ -227,6 +283,7 @@ def main() -> int:
 
     extra = {"gemv_e4m3_16384_cold_first_series_us": round(cold_us, 2)}   # same kernel, first series: no warm-up, first-launch cost included
     rl = {}                                                               # roofline records of the other HBM-bound workloads
+    arl = {}                                                              # roofline records of the matrix-core-bound workloads (attention)
     if not args.no_extra:
         # cache-resident figure (one matrix re-used): reported separately, never the headline
         one = mats["E4M3"][0]
@@ -239,19 +296,20 @@ def main() -> int:
 
         def gemv_grid(mode):
             bufs = mats[mode]
-            for (Ms, Ks) in ((4096, 4096), (8192, 8192), (16384, 8192)):
-                words = Ms * Ks // 4
-                per = (M * K // 4) // words
-                views = [b[i * words:(i + 1) * words] for b in bufs for i in range(per)]
-                vp = feather.pack_fp8_tensor(v16[:Ks], mode=mode)
-                call = lambda i: feather.gemv(views[i % len(views)], vp, original_shape=(Ms, Ks), mode=mode)
-                us = gpu_time_us(call, args.steps, args.warmup, sync, 10.0)
-                if us < 12.0:                                   # shorter than the host's per-call cost: time the device alone
-                    us = min(us, gpu_time_graph_us(call, max(16, len(views)), sync))
-                key = f"gemv_{mode.lower()}_{Ms}x{Ks}" if Ms != Ks else f"gemv_{mode.lower()}_{Ms}"
-                extra[key + "_us"] = round(us, 2)
-                extra[key + "_GBps"] = round((Ms * Ks + Ks + 4 * Ms) / us / 1e3, 1)
-                rl[key] = roofline_record(ttab, key, f"gemv_fp8_kernel<{mode}>", Ms * Ks + Ks + 4 * Ms, us)
+            for Ms in (4096, 8192, 16384):
+                for Ks in (4096, 8192, 16384):
+                    if Ms == M and Ks == K:
+                        continue                                 # 16384^2 is the headline (E4M3) / its own series (E5M2)
+                    words = Ms * Ks // 4
+                    per = (M * K // 4) // words
+                    views = [b[i * words:(i + 1) * words] for b in bufs for i in range(per)]
+                    vp = feather.pack_fp8_tensor(v16[:Ks], mode=mode)
+                    call = lambda i: feather.gemv(views[i % len(views)], vp, original_shape=(Ms, Ks), mode=mode)
+                    us, how = gpu_time_auto_us(call, min(64, len(views)), args.steps, args.warmup, sync, 10.0)
+                    key = f"gemv_{mode.lower()}_{Ms}x{Ks}" if Ms != Ks else f"gemv_{mode.lower()}_{Ms}"
+                    extra[key + "_us"] = round(us, 2)
+                    extra[key + "_GBps"] = round((Ms * Ks + Ks + 4 * Ms) / us / 1e3, 1)
+                    rl[key] = roofline_record(ttab, key, f"gemv_fp8_kernel<{mode}>", Ms * Ks + Ks + 4 * Ms, us, timing=how)
             # batched GEMV: the rotating matrices against 32 vectors (weights streamed once per batch)
             xb = feather.pack_fp8_tensor(randn(32, K).half(), mode=mode)
             us = gpu_time_us(lambda i: gemv_fp8_batched_acc_fp32_gpu(bufs[i % NBUF], xb, (M, K), 32, mode), 50, 10, sync)
@@ -270,7 +328,8 @@ def main() -> int:
         extra["gemv_e5m2_16384_hbm_frac"] = round(gemv_bytes / us / 1e3 / HBM_PEAK_GBS, 4)
         rl["gemv_e5m2_16384"] = roofline_record(ttab, "gemv_e5m2_16384", "gemv_fp8_kernel<E5M2>", gemv_bytes, us)
         gemv_grid("E5M2")
-        # dot, n = 2^24 (E4M3): rotate through the big buffers
+        # dot, n = 2^24: rotate through the big buffers (64 distinct operands of 16 MiB)
+        from feather_amd.routines.dot import dot_fp16_acc_fp32_gpu
         n = 1 << 24
         xs = [b[i * (n // 4):(i + 1) * (n // 4)] for b in mats["E5M2"] for i in range(16)]
         for mode in ("E4M3", "E5M2"):
@@ -281,12 +340,29 @@ def main() -> int:
             extra[f"dot_{mode.lower()}_2p24_us"] = round(us, 2)
             extra[f"dot_{mode.lower()}_2p24_GBps"] = round((2 * n + 4) / us / 1e3, 1)
             rl[f"dot_{mode.lower()}_2p24"] = roofline_record(ttab, f"dot_{mode.lower()}_2p24", f"dot_kernel<{mode}> + dot_finish_kernel",
-                                                              2 * n + 4, us, launches_per_call=2)
+                                                              2 * n + 4, us, launches_per_call=2, timing="graph")
+        # FP16-packed dot (reference dot_fp16_acc_fp32_gpu, benchmark/bench_dot.py:138-160), n = 2^24 elements: 2 B per
+        # element and operand, operands of 32 MiB taken from the same rotating buffers
+        xh = [b[i * (n // 2):(i + 1) * (n // 2)] for b in mats["E5M2"] for i in range(8)]
+        us = gpu_time_graph_us(lambda i: dot_fp16_acc_fp32_gpu(xh[(2 * i) % 32], xh[(2 * i + 1) % 32]), 32, sync)
+        extra["dot_fp16_2p24_us"] = round(us, 2)
+        extra["dot_fp16_2p24_GBps"] = round((4 * n + 4) / us / 1e3, 1)
+        rl["dot_fp16_2p24"] = roofline_record(ttab, "dot_fp16_2p24", "dot_kernel<FP16> + dot_finish_kernel", 4 * n + 4, us,
+                                              launches_per_call=2, timing="graph")
+        # the largest size of the reference harness (benchmark/bench_dot.py:15), n = 1 500 000
+        nh = 1_500_000
+        for kind, words, call in (("e5m2", nh // 4, lambda a, b: feather.dot(a, b, mode="E5M2")),
+                                  ("fp16", nh // 2, lambda a, b: dot_fp16_acc_fp32_gpu(a, b))):
+            ops = [mats["E5M2"][0][i * words:(i + 1) * words] for i in range(32)]
+            us = gpu_time_graph_us(lambda i: call(ops[(2 * i) % 32], ops[(2 * i + 1) % 32]), 32, sync)
+            extra[f"dot_{kind}_1500000_us"] = round(us, 2)
         # dot, n = 16384 (one workgroup, one launch: latency bound)
         xs_s = [x[:4096] for x in xs]
         for mode in ("E4M3", "E5M2"):
             us = gpu_time_graph_us(lambda i: feather.dot(xs_s[(2 * i) % 64], xs_s[(2 * i + 1) % 64], mode=mode), 32, sync)
             extra[f"dot_{mode.lower()}_16384_us"] = round(us, 2)
+        extra["dot_timing"] = "graph replay of 32 captured calls (device time; a Python call costs 8-11 us on the host)"
+        del xh
         # pack throughput (2 B in + 1 B out per element)
         src = randn(8192, 16384).half()
         for mode in ("E5M2", "E4M3"):
@@ -310,6 +386,7 @@ def main() -> int:
         torch.cuda.empty_cache()
         # flash attention, B4 H16 d64, E5M2, vs fp16 SDPA on the same GPU (both sides get WARM_MS of
         # back-to-back warm-up calls: the first tens of milliseconds of a series run below the sustained clock)
+        busy = load_mfma_busy()
         for L in (4096, 8192):
             B, H, d = 4, 16, 64
             qkv16 = [randn(B, H, L, d).half() for _ in range(3)]
@@ -317,25 +394,33 @@ def main() -> int:
             us = gpu_time_us(lambda i: feather.flash_attention_fp8_e5m2_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4),
                              10, 10, sync, warm_ms)
             flops = 4.0 * B * H * L * L * d
-            extra[f"flash_attn_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
-            extra[f"flash_attn_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / us / 1e6, 1)
-            extra[f"flash_attn_e5m2_b4h16_d64_L{L}_mfma_frac"] = round(flops / us / 1e6 / MFMA_PEAK_F16_TFLOPS, 4)
             us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync, warm_ms)
+            key = f"flash_attn_e5m2_b4h16_d64_L{L}"
+            extra[key + "_us"] = round(us, 1)
+            extra[key + "_TFLOPs"] = round(flops / us / 1e6, 1)
+            extra[key + "_mfma_frac"] = round(flops / us / 1e6 / MFMA_PEAK_F16_TFLOPS, 4)
             extra[f"sdpa_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
+            # Q K^T (half the flops) runs on the bf8 matrix instruction at the FP8 rate, P V on the fp16 one
+            arl[key] = mfma_record(busy, key, "flash_attn64_wide_kernel<E5M2>", flops, us, 0.5, us_sdpa)
             if L == 8192:   # causal prefill (half the flops) vs causal fp16 SDPA
                 us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
                                                                                     mode="E5M2", causal=True), 10, 10, sync, warm_ms)
-                extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_us"] = round(us, 1)
-                extra[f"flash_attn_causal_e5m2_b4h16_d64_L{L}_TFLOPs"] = round(flops / 2 / us / 1e6, 1)
                 us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16, is_causal=True),
                                       10, 10, sync, warm_ms)
+                key = f"flash_attn_causal_e5m2_b4h16_d64_L{L}"
+                extra[key + "_us"] = round(us, 1)
+                extra[key + "_TFLOPs"] = round(flops / 2 / us / 1e6, 1)
                 extra[f"sdpa_causal_fp16_b4h16_d64_L{L}_us"] = round(us_sdpa, 1)
+                arl[key] = mfma_record(busy, key, "flash_attn64_wide_kernel<E5M2, causal>", flops / 2, us, 0.5, us_sdpa)
             if L == 8192:   # the same shape with E4M3 codes (fp16 score product: the E4M3 kernel decode is not the matrix core's format)
                 pk4 = [feather.pack_fp8_tensor(t, mode="E4M3").view(B, H, L, d // 4) for t in qkv16]
                 us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk4[0], pk4[1], pk4[2], L, d // 4, mode="E4M3"),
                                  10, 10, sync, warm_ms)
-                extra[f"flash_attn_e4m3_b4h16_d64_L{L}_us"] = round(us, 1)
-                extra[f"flash_attn_e4m3_b4h16_d64_L{L}_TFLOPs"] = round(flops / us / 1e6, 1)
+                key = f"flash_attn_e4m3_b4h16_d64_L{L}"
+                extra[key + "_us"] = round(us, 1)
+                extra[key + "_TFLOPs"] = round(flops / us / 1e6, 1)
+                us_sdpa = extra[f"sdpa_fp16_b4h16_d64_L{L}_us"]
+                arl[key] = mfma_record(busy, key, "flash_attn64_wide_kernel<E4M3>", flops, us, 0.0, us_sdpa)
                 del pk4
             del qkv16, pk
         # wide heads: B1 H8, d = 256 / 512, E4M3, vs fp16 SDPA
@@ -345,10 +430,12 @@ def main() -> int:
             pk = [feather.pack_fp8_tensor(t, mode="E4M3").view(B, H, L, d // 4) for t in qkv16]
             us = gpu_time_us(lambda i: feather.flash_attention_fp8_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4,
                                                                                 mode="E4M3"), 10, 10, sync, warm_ms)
-            extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_us"] = round(us, 1)
-            extra[f"flash_attn_e4m3_b1h8_d{d}_L{L}_TFLOPs"] = round(4.0 * B * H * L * L * d / us / 1e6, 1)
+            key = f"flash_attn_e4m3_b1h8_d{d}_L{L}"
+            extra[key + "_us"] = round(us, 1)
+            extra[key + "_TFLOPs"] = round(4.0 * B * H * L * L * d / us / 1e6, 1)
             us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync, warm_ms)
             extra[f"sdpa_fp16_b1h8_d{d}_L{L}_us"] = round(us_sdpa, 1)
+            arl[key] = mfma_record(busy, key, f"flash_attn_kernel<{d}, E4M3>", 4.0 * B * H * L * L * d, us, 0.0, us_sdpa)
             del qkv16, pk
         torch.cuda.empty_cache()
         # paged-attention decode, 32 sequences x 32 query heads over 4 KV heads, d=64, E4M3, blocks of 16
@@ -356,29 +443,33 @@ def main() -> int:
         from feather_amd.routines.paged_attention import paged_attention_fp8_acc_fp32_gpu
         n_seq, Hq, Hkv, d, bs, cmax = 32, 32, 4, 64, 16, 4096
         nblk = n_seq * cmax // bs
-        kc, vc = (feather.pack_fp8_tensor(randn(nblk * Hkv * bs * d).half(), mode="E4M3").view(nblk, Hkv, bs, d // 4)
-                  for _ in range(2))
+        NKV = 4                                                  # K/V cache pairs rotated: 4 x 67 MB > the 256 MB Infinity Cache
+        caches = [tuple(feather.pack_fp8_tensor(randn(nblk * Hkv * bs * d).half(), mode="E4M3").view(nblk, Hkv, bs, d // 4)
+                        for _ in range(2)) for _ in range(NKV)]
+        kc, vc = caches[0]
         qp = feather.pack_fp8_tensor(randn(n_seq * Hq * d).half(), mode="E4M3").view(n_seq, Hq, d // 4)
         bt = torch.randperm(nblk, generator=g, device=dev).to(torch.int32).view(n_seq, cmax // bs)
         for c in (512, 4096):
             cl = torch.full((n_seq,), c, dtype=torch.int32, device=dev)
-            us = gpu_time_graph_us(lambda i: paged_attention_fp8_acc_fp32_gpu(qp, kc, vc, bt, cl, mode="E4M3",
-                                                                              max_context_len=c), 16, sync)
+            us = gpu_time_graph_us(lambda i: paged_attention_fp8_acc_fp32_gpu(qp, caches[i % NKV][0], caches[i % NKV][1], bt, cl,
+                                                                              mode="E4M3", max_context_len=c), 16, sync)
             extra[f"paged_attn_e4m3_s32_h32kv4_d64_ctx{c}_us"] = round(us, 2)
             extra[f"paged_attn_e4m3_s32_h32kv4_d64_ctx{c}_GBps"] = round(2 * n_seq * Hkv * d * c / us / 1e3, 1)
             rl[f"paged_attn_e4m3_ctx{c}"] = roofline_record(
                 ttab, f"paged_attn_e4m3_ctx{c}", "paged_attn_split_kernel<64, E4M3>" + (" + paged_attn_merge_kernel" if c > 512 else ""),
-                2 * n_seq * Hkv * d * c + n_seq * Hq * d * 5, us, launches_per_call=2 if c > 512 else 1)
+                2 * n_seq * Hkv * d * c + n_seq * Hq * d * 5, us, launches_per_call=2 if c > 512 else 1, timing="graph",
+                note=f"{NKV} K/V cache pairs rotated" + ("" if c > 512 else
+                     ": at this context a call reads 8 MB, so the four caches together (34 MB) stay in the 256 MB Infinity Cache"))
         # prefill -> paged cache: 32 sequences x 2048 rows x 4 KV heads of packed K and V (1 B in + 1 B out per code)
         from feather_amd.routines.paged_attention import paged_cache_write
         rows = n_seq * 2048
         ksrc, vsrc = (feather.pack_fp8_tensor(randn(Hkv * rows * d).half(), mode="E4M3").view(Hkv, rows, d // 4)
                       for _ in range(2))
         cu = torch.arange(0, rows + 1, 2048, dtype=torch.int32, device=dev)
-        us = gpu_time_graph_us(lambda i: paged_cache_write(ksrc, vsrc, kc, vc, bt, cu, mode="E4M3"), 16, sync)
+        us = gpu_time_graph_us(lambda i: paged_cache_write(ksrc, vsrc, kc, vc, bt, cu, mode="E4M3"), 16, sync)   # device time (graph replay)
         extra["paged_cache_write_e4m3_s32_L2048_kv4_d64_us"] = round(us, 2)
         extra["paged_cache_write_e4m3_s32_L2048_kv4_d64_GBps"] = round(4 * Hkv * rows * d / us / 1e3, 1)
-        del kc, vc, qp, ksrc, vsrc
+        del kc, vc, caches, qp, ksrc, vsrc
         torch.cuda.empty_cache()
         # decode step of a TinyLlama-1.1B-shaped model (random weights), contexts 512..4095: batch 32 in E4M3
         # (the configuration of the metric), then E5M2 and batch 64 for comparison
@@ -416,11 +507,32 @@ def main() -> int:
                "pack_us": round(r["pack_s"] * 1e6, 1), "decode_us": round(r["decode_s"] * 1e6, 1),
                "compute_us": round(r["compute_s"] * 1e6, 1), "cpu_count": r["cpu_count"]}
         # second half of the metric: pack + decode + fp32 SDPA per head (B4 H16 d=64 L=8192, E5M2), 16 of the 64 heads timed
-        ra = cpu_baseline.attention_baseline(64, 8192, 64, "E5M2", sample_heads=16, repeats=3)
-        cpu["flash_attn_e5m2_b4h16_d64_L8192"] = {
-            "value": round(ra["total_s"] * 1e6, 1), "unit": "us", "cores": ra["cores"], "kind": "port",
-            "sample": ra["sample"] + "; pack + decode (LUT gather) + fp32 SDPA per head, summed, median of 3",
-            "pack_us": round(ra["pack_s"] * 1e6, 1), "decode_and_sdpa_us": round(ra["compute_s"] * 1e6, 1)}
+        def attn_leg(heads, L, d, mode, sample_heads, repeats):
+            ra = cpu_baseline.attention_baseline(heads, L, d, mode, sample_heads=sample_heads, repeats=repeats)
+            return {"value": round(ra["total_s"] * 1e6, 1), "unit": "us", "cores": ra["cores"], "kind": "port",
+                    "sample": ra["sample"] + f"; pack + decode (LUT gather) + fp32 SDPA per head, summed, median of {repeats}",
+                    "pack_us": round(ra["pack_s"] * 1e6, 1), "decode_and_sdpa_us": round(ra["compute_s"] * 1e6, 1)}
+        cpu["flash_attn_e5m2_b4h16_d64_L8192"] = attn_leg(64, 8192, 64, "E5M2", 16, 3)
+        if not args.no_extra:
+            # the other configurations, each a bounded sample of the same workload (the scaling is in `sample`)
+            r1 = cpu_baseline.gemv_baseline(8192, 8192, "E5M2", sample_rows=8192, repeats=5)
+            cpu["gemv_e5m2_8192"] = {"value": round(r1["total_s"] * 1e6, 1), "unit": "us", "cores": r1["cores"], "kind": "port",
+                                     "sample": r1["sample"], "pack_us": round(r1["pack_s"] * 1e6, 1),
+                                     "decode_us": round(r1["decode_s"] * 1e6, 1), "compute_us": round(r1["compute_s"] * 1e6, 1)}
+            rd = cpu_baseline.dot_baseline(1 << 24, "E4M3", repeats=5)
+            cpu["dot_e4m3_2p24"] = {"value": round(rd["total_s"] * 1e6, 1), "unit": "us", "cores": rd["cores"], "kind": "port",
+                                    "sample": rd["sample"], "pack_us": round(rd["pack_s"] * 1e6, 1),
+                                    "decode_us": round(rd["decode_s"] * 1e6, 1), "compute_us": round(rd["compute_s"] * 1e6, 1)}
+            cpu["flash_attn_e5m2_b4h16_d64_L4096"] = attn_leg(64, 4096, 64, "E5M2", 16, 3)
+            cpu["flash_attn_e4m3_b1h8_d256_L4096"] = attn_leg(8, 4096, 256, "E4M3", 8, 3)
+            cpu["flash_attn_e4m3_b1h8_d512_L8192"] = attn_leg(8, 8192, 512, "E4M3", 2, 3)
+            from feather_amd.routines.decode import TINYLLAMA_1_1B
+            gcpu = torch.Generator().manual_seed(5)
+            rs = cpu_baseline.decode_step_baseline(TINYLLAMA_1_1B, 32, torch.randint(512, 4096, (32,), generator=gcpu).tolist(),
+                                                   "E4M3", sample_layers=2, repeats=3)
+            cpu["decode_tinyllama_b32_e4m3"] = {"value": round(rs["total_s"] * 1e3, 2), "unit": "ms per step", "cores": rs["cores"],
+                                                "kind": "port", "sample": rs["sample"],
+                                                "tokens_per_s": round(32 / rs["total_s"], 1)}
 
     line = {
         "metric": "packed-FP8 GEMV us (16384^2, E4M3, FP32 accumulate)",
@@ -431,9 +543,13 @@ def main() -> int:
                                "sources with 1% of entries x1e-3, packed 4 codes per 32-bit word; 4 distinct "
                                "matrices (1 GiB) rotated",
                    "M": M, "K": K, "mode": "E4M3", "buffers": NBUF, "clock_prewarm_launches": PREWARM, "gate_launches": GATE},
-        "roofline": dict(headline, avg_launch_us=round(kern_us, 3)),
+        # the headline kernel's record; the second half of the metric (flash attention d = 64, L = 8192) is the nested
+        # matrix-core record, the other attention workloads are in extra.roofline_mfma
+        "roofline": dict(headline, avg_launch_us=round(kern_us, 3),
+                         **({"flash_attn_e5m2_b4h16_d64_L8192": arl["flash_attn_e5m2_b4h16_d64_L8192"]}
+                            if "flash_attn_e5m2_b4h16_d64_L8192" in arl else {})),
         "cpu_baseline": cpu,
-        "extra": dict(extra, roofline=rl),
+        "extra": dict(extra, roofline=rl, roofline_mfma=arl),
     }
     print(json.dumps(line))
     return 0

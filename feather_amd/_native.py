@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libfeather_hip.so")
 
 OK, EINVAL, EMODE, ESHAPE, ELAUNCH = 0, -1, -2, -3, -4
-ABI_VERSION = 10300   # FEATHER_HIP_VERSION of the include/feather_hip.h these signatures were written against
+ABI_VERSION = 10400   # FEATHER_HIP_VERSION of the include/feather_hip.h these signatures were written against
 E5M2, E4M3 = 0, 1
 ROUND_RNE, ROUND_TRUNC = 0, 1
 SEM_KERNEL, SEM_IEEE = 0, 1
@@ -42,6 +42,8 @@ SIGNATURES = {
     "feather_dot_fp8": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _vp]),
     "feather_dot_fp16": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _vp]),
     "feather_flash_attn_fp8": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _f32, _i32, _vp]),
+    "feather_flash_attn_fp8_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _f32, _i32, _vp]),
+    "feather_flash_attn_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "feather_flash_attn_fp8_varlen": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _f32,
                                              _i32, _vp]),
     "feather_paged_cache_write": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,

@@ -80,12 +80,18 @@ __device__ __forceinline__ half8_t dec8(uint32_t w0, uint32_t w1) {
 //         one worked).  A group of 16 keys multiplies P and V on the 16x16x16 MFMA.  Group 0 always has
 //         key 0, so its running maximum is finite whenever the sequence has a key; not combined with
 //         the causal mask.
-template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC, int WAVES = 4, int KSPLIT = 1>
+// ZS  the key loop is cut into n_kchunks ranges of kchunk_keys keys (a multiple of BN, every range starting
+//     below L) that go to separate workgroups, for grids that would leave most CUs idle: workgroup
+//     (tile, z) scores range z and writes its unnormalised accumulators, reference point and row sum to
+//     `part` ([z][row][D] floats, then [z][row] pairs (m, l)); flash_attn_merge_kernel combines the ranges.
+//     Fixed-length heads only.
+template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC, int WAVES = 4, int KSPLIT = 1, bool ZS = false>
 __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     const uint32_t *__restrict__ q, const uint32_t *__restrict__ k, const uint32_t *__restrict__ v,
     float *__restrict__ out, int L, int n_heads, int kv_group, int tiles_per_head, float scale_log2e,
     int keys_scored, int mask_tail, const int32_t *__restrict__ cu_seqlens, int tiles_per_seq, int total_rows,
-    int causal) {
+    int causal, float *__restrict__ part, int kchunk_keys, int n_kchunks) {
+    static_assert(!(ZS && VC), "key ranges over workgroups are for fixed-length heads");
     constexpr int DW = D / 4;              // packed words per row
     // E5M2 codes ARE the bf8 operand format of the matrix core: the score product runs on
     // v_mfma_f32_16x16x32_bf8_bf8 straight from the packed bytes (exact products, fp32 accumulation,
@@ -125,6 +131,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     int bid = blockIdx.x;
     const int total = gridDim.x;
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
+    int zchunk = 0;
+    if constexpr (ZS) {   // the key ranges of a query tile are neighbours in this order: same XCD, same L2
+        zchunk = bid % n_kchunks;
+        bid /= n_kchunks;
+    }
     const int head = bid / tiles_per_head;
     int tile = bid % tiles_per_head;
     const int kv_head = head / kv_group;
@@ -262,12 +273,14 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         }
     };
 
-    prefetch(0);
+    const int key_begin = ZS ? zchunk * kchunk_keys : 0;
+    const int key_end = ZS ? min(keys_scored, key_begin + kchunk_keys) : keys_scored;
+    prefetch(key_begin);
     stage(0);
-    if (BN < keys_scored) prefetch(BN);
+    if (key_begin + BN < key_end) prefetch(key_begin + BN);
     __syncthreads();
     int cur = 0;
-    for (int key0 = 0; key0 < keys_scored; key0 += BN, cur ^= 1) {
+    for (int key0 = key_begin; key0 < key_end; key0 += BN, cur ^= 1) {
         // tile i+1 goes to the other buffer (its readers passed the barrier that ended the previous
         // iteration) and tile i+2 into registers, both off the critical path of this tile's math
         // At d = 512 the two waves that share a SIMD (w and w + 4 of an eight-wave workgroup) run this
@@ -275,9 +288,9 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         // reads and MFMAs, and in lock step the pair wants the same unit at the same time (-2..5 % time;
         // the narrower heads lose 1-4 % with it, their staging is a smaller share of a tile).
         const bool math_first = WAVES == 8 && D >= 512 && wave >= 4;
-        if (!math_first && key0 + BN < keys_scored) {
+        if (!math_first && key0 + BN < key_end) {
             stage(cur ^ 1);
-            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
+            if (key0 + 2 * BN < key_end) prefetch(key0 + 2 * BN);
         }
         const _Float16 *k_lds = lds + cur * kBufHalfs;
         const _Float16 *vt_lds = k_lds + BN * KS;
@@ -378,6 +391,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
                     }
                 }
             }
+            mfma_settle<SB * GKB16>(&s[0][0]);   // the softmax's first readers are asm statements
 #pragma unroll
             for (int b = 0; b < SB; b++) softmax_block(b0 + b, s[b], pf[b0 + b]);
         }
@@ -412,9 +426,9 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         }
         }
         }   // !skip
-        if (math_first && key0 + BN < keys_scored) {
+        if (math_first && key0 + BN < key_end) {
             stage(cur ^ 1);
-            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
+            if (key0 + 2 * BN < key_end) prefetch(key0 + 2 * BN);
         }
         __syncthreads();  // tile i+1 is visible; every wave is done reading tile i
     }
@@ -467,6 +481,24 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
         if (kgroup != 0) return;
     }
 
+    if constexpr (ZS) {
+        // ---- epilogue of a key range: unnormalised accumulators, reference point and row sum
+        const int64_t rows_total = (int64_t)n_heads * L;
+        float *ph = part + ((int64_t)zchunk * rows_total + q_row0) * D;
+        float *ml = part + (int64_t)n_kchunks * rows_total * D + ((int64_t)zchunk * rows_total + q_row0) * 2;
+#pragma unroll
+        for (int b = 0; b < QB; b++) {
+            int row = q0 + 16 * b + j;
+            if (row < L) {
+#pragma unroll
+                for (int d = 0; d < DB; d++)
+                    *reinterpret_cast<float4_t *>(ph + (int64_t)row * D + 16 * d + 4 * kb) = o[b][d];
+                if (kb == 0) *reinterpret_cast<float2v_t *>(ml + (int64_t)row * 2) = float2v_t{m_run[b], o[b][DB][0]};
+            }
+        }
+        return;
+    }
+
     // ---- epilogue: finish the row sums, normalise, store [q][dd]
     float *oh = out + q_row0 * D;
 #pragma unroll
@@ -480,6 +512,41 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
             }
         }
     }
+}
+
+// Combines the key ranges of flash_attn_kernel<..., ZS = true>: one thread per (row, four dims).  Range z of a row
+// holds O_z = sum_k 2^((s_k - m_z) c) V_k and l_z = sum_k 2^((s_k - m_z) c); with m = max_z m_z the row is
+// sum_z 2^((m_z - m) c) O_z / sum_z 2^((m_z - m) c) l_z, added in range order.
+__global__ __launch_bounds__(256) void flash_attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out,
+                                                               int64_t rows_total, int dq, int n_kchunks,
+                                                               float scale_log2e) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= rows_total * dq) return;
+    const int64_t row = idx / dq;
+    const float2v_t *ml = reinterpret_cast<const float2v_t *>(part + (int64_t)n_kchunks * rows_total * dq * 4);
+    const float4_t *po = reinterpret_cast<const float4_t *>(part);
+    float2v_t mlz[4];
+    float4_t oz[4];
+#pragma unroll
+    for (int z = 0; z < 4; z++)
+        if (z < n_kchunks) {
+            mlz[z] = ml[z * rows_total + row];
+            oz[z] = po[z * rows_total * dq + idx];
+        }
+    float m = mlz[0][0];
+#pragma unroll
+    for (int z = 1; z < 4; z++)
+        if (z < n_kchunks) m = fmaxf(m, mlz[z][0]);
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    float l = 0.f;
+#pragma unroll
+    for (int z = 0; z < 4; z++)
+        if (z < n_kchunks) {
+            const float w = mlz[z][0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mlz[z][0] - m) * scale_log2e);
+            acc += oz[z] * w;
+            l += mlz[z][1] * w;
+        }
+    reinterpret_cast<float4_t *>(out)[idx] = acc / l;
 }
 
 // ---- d = 64, E5M2: the FP8-rate kernel -------------------------------------------------------------
@@ -838,10 +905,18 @@ struct AttnArgs {
     const void *cu_seqlens;
     int64_t n_seq, max_seqlen, total_rows;
     int causal;
+    void *ws;           // optional device workspace for key ranges over workgroups (fixed-length heads)
+    int64_t ws_bytes;
 };
 
-template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC, int WAVES = 4, int KSPLIT = 1>
-static int launch_attn(const AttnArgs &a, hipStream_t s) {
+constexpr int kMaxKeyChunks = 4;
+// Bytes of workspace that n_kchunks key ranges of n_heads * L rows need: accumulators, then (m, l) pairs.
+static int64_t key_chunk_ws_bytes(int64_t n_heads, int64_t L, int64_t d, int n_kchunks) {
+    return n_kchunks * n_heads * L * (d + 2) * 4;
+}
+
+template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC, int WAVES = 4, int KSPLIT = 1, bool ZS = false>
+static int launch_attn(const AttnArgs &a, hipStream_t s, int n_kchunks = 1) {
     constexpr int QT = 16 * QB * WAVES / KSPLIT;
     constexpr int KS = MODE == FEATHER_E5M2 ? (D + 16) / 2 : D + 8;   // K row pitch in fp16 units, as in the kernel
     constexpr size_t lds = (size_t)(BN * KS + D * BN) * 2 * 2;        // two (K, V^T) buffers
@@ -853,18 +928,27 @@ static int launch_attn(const AttnArgs &a, hipStream_t s) {
     if (blocks == 0) return FEATHER_OK;
     // the reference scores whole 64-key tiles (zero rows past L); otherwise only tiles of BN up to L
     int64_t keys_scored = a.tail == FEATHER_TAIL_REFERENCE ? (L + 63) / 64 * 64 : (L + BN - 1) / BN * BN;
-    auto kern = flash_attn_kernel<D, MODE, QB, SB, BN, OCC, VC, WAVES, KSPLIT>;
+    auto kern = flash_attn_kernel<D, MODE, QB, SB, BN, OCC, VC, WAVES, KSPLIT, ZS>;
+    // key ranges: whole tiles, every range starting below the last scored key
+    const int64_t n_tiles_k = keys_scored / BN;
+    const int64_t kchunk_keys = (n_tiles_k + n_kchunks - 1) / n_kchunks * BN;
+    if (ZS) n_kchunks = (int)((keys_scored + kchunk_keys - 1) / kchunk_keys);
     static unsigned long long lds_raised = 0;   // per instantiation, one bit per device
     hipError_t e = raise_lds_limit(reinterpret_cast<const void *>(kern), lds, lds_raised);
     FEATHER_CHECK(e == hipSuccess, FEATHER_ELAUNCH, "feather_flash_attn_fp8: cannot raise LDS limit: %s",
                   hipGetErrorString(e));
     const float log2e = 1.4426950408889634f;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * WAVES), lds, s, (const uint32_t *)a.q,
-                       (const uint32_t *)a.k, (const uint32_t *)a.v, (float *)a.out, (int)L, (int)a.n_heads,
-                       (int)a.kv_group, (int)tiles, a.scale * log2e, (int)keys_scored,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(blocks * (ZS ? n_kchunks : 1))), dim3(64 * WAVES), lds, s,
+                       (const uint32_t *)a.q, (const uint32_t *)a.k, (const uint32_t *)a.v, (float *)a.out, (int)L,
+                       (int)a.n_heads, (int)a.kv_group, (int)tiles, a.scale * log2e, (int)keys_scored,
                        a.tail == FEATHER_TAIL_MASK ? 1 : 0, (const int32_t *)a.cu_seqlens, tiles_per_seq,
-                       (int)a.total_rows, a.causal);
-    return check_launch("feather_flash_attn_fp8");
+                       (int)a.total_rows, a.causal, (float *)a.ws, (int)kchunk_keys, n_kchunks);
+    int rc = check_launch("feather_flash_attn_fp8");
+    if (!ZS || rc != FEATHER_OK) return rc;
+    const int64_t rows_total = a.n_heads * L, quads = rows_total * (D / 4);
+    hipLaunchKernelGGL(flash_attn_merge_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s,
+                       (const float *)a.ws, (float *)a.out, rows_total, D / 4, n_kchunks, a.scale * log2e);
+    return check_launch("feather_flash_attn_fp8 (merge of the key ranges)");
 }
 
 template <int MODE, bool VC, int WAVES, int OCC>
@@ -893,9 +977,31 @@ static int launch_attn64_wide(const AttnArgs &a, hipStream_t s) {
 // eight waves (twice the queries per staged tile, two waves per SIMD from one workgroup to overlap
 // the barrier-separated phases) are faster wherever the coarser grid still covers the chip's 256 CUs;
 // d = 256 takes eight waves at every length.
+// Key ranges over workgroups (fixed-length, non-causal heads of 128 dims and more): the number of ranges the
+// finest workgroup shape of head dim d is cut into, doubled while the grid still fits the 256 CUs in one pass
+// and a range keeps at least four key tiles.  1 = the plain kernel.
+static int pick_key_chunks(int64_t d, int64_t n_heads, int64_t L) {
+    int64_t queries, bn;
+    switch (d) {
+        case 128: queries = 128; bn = 64; break;
+        case 256: queries = 64; bn = 64; break;
+        case 512: queries = 64; bn = 32; break;
+        default: return 1;
+    }
+    const int64_t wgs = (L + queries - 1) / queries * n_heads, tiles = (L + bn - 1) / bn;
+    int z = 1;
+    while (z < kMaxKeyChunks && wgs * z * 2 <= 256 && tiles / (z * 2) >= 4) z *= 2;
+    return z;
+}
+
 template <int MODE, bool VC>
 static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
     const int64_t rows = VC ? a.max_seqlen : a.L, seqs = VC ? a.n_seq : 1;
+    int zs = 1;
+    if (!VC && a.ws) {
+        zs = pick_key_chunks(d, a.n_heads, a.L);
+        while (zs > 1 && a.ws_bytes < key_chunk_ws_bytes(a.n_heads, a.L, d, zs)) zs /= 2;   // a smaller workspace: fewer ranges
+    }
     auto fills_chip = [&](int64_t queries_per_group) {
         return (rows + queries_per_group - 1) / queries_per_group * seqs * a.n_heads >= 256;
     };
@@ -911,6 +1017,8 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
             if (!a.causal && fills_chip(512)) return launch_attn64_wide<MODE, VC, 8, 1>(a, s);
             return launch_attn64_wide<MODE, VC, 4, 2>(a, s);
         case 128:
+            if constexpr (!VC)
+                if (zs > 1) return launch_attn<128, MODE, 2, 2, 64, 2, false, 4, 1, true>(a, s, zs);
             if (fills_chip(256)) return launch_attn<128, MODE, 2, 2, 64, 1, VC, 8>(a, s);
             return launch_attn<128, MODE, 2, 2, 64, 2, VC>(a, s);
         case 256: {
@@ -919,6 +1027,8 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
             // every key tile (2.9 us); B = 128 queries, eight waves of 16 (3.2 us); C = 256 queries,
             // eight waves of 32 on 32-key tiles, which halves the LDS reads per query that bound this
             // head dim (4.6 us; L = 8192: 792 -> 640 us against B).  Pick by rounds over the 256 CUs x cost.
+            if constexpr (!VC)
+                if (zs > 1) return launch_attn<256, MODE, 1, 1, 64, 1, false, 8, 2, true>(a, s, zs);
             const int64_t ra = rounds(64), rb = rounds(128), rc = rounds(256);
             if (!a.causal && ra * 29 <= rb * 32 && ra * 29 <= rc * 46) return launch_attn<256, MODE, 1, 1, 64, 1, VC, 8, 2>(a, s);
             if (rc * 46 < rb * 32 || fills_chip(256)) return launch_attn<256, MODE, 2, 2, 32, 1, VC, 8>(a, s);
@@ -927,6 +1037,8 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
         case 512: {
             // A = 64 queries, two wave groups of 16 keys per 32-key tile (3.1 us per tile of a
             // workgroup's loop); B = 128 queries, eight waves (3.5 us)
+            if constexpr (!VC)
+                if (zs > 1) return launch_attn<512, MODE, 1, 1, 32, 1, false, 8, 2, true>(a, s, zs);
             const int64_t ra = rounds(64), rb = rounds(128);
             if (!a.causal && ra * 31 <= rb * 35) return launch_attn<512, MODE, 1, 1, 32, 1, VC, 8, 2>(a, s);
             if (fills_chip(128) || !a.causal) return launch_attn<512, MODE, 1, 1, 32, 1, VC, 8>(a, s);
@@ -941,11 +1053,25 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
 
 using namespace feather;
 
+extern "C" int64_t feather_flash_attn_workspace_bytes(int64_t n_heads, int64_t L, int64_t d) {
+    if (n_heads <= 0 || L <= 0 || L >= (1ll << 30)) return 0;
+    const int z = pick_key_chunks(d, n_heads, L);
+    return z > 1 ? key_chunk_ws_bytes(n_heads, L, d, z) : 0;
+}
+
 extern "C" int feather_flash_attn_fp8(const void *q, const void *k, const void *v, void *out_f32, int64_t n_heads,
                                       int64_t L, int64_t d, int64_t kv_group, int mode, float scale, int tail,
                                       void *stream) {
+    return feather_flash_attn_fp8_ws(q, k, v, out_f32, nullptr, 0, n_heads, L, d, kv_group, mode, scale, tail, stream);
+}
+
+extern "C" int feather_flash_attn_fp8_ws(const void *q, const void *k, const void *v, void *out_f32, void *workspace,
+                                         int64_t workspace_bytes, int64_t n_heads, int64_t L, int64_t d,
+                                         int64_t kv_group, int mode, float scale, int tail, void *stream) {
     FEATHER_CHECK(mode == FEATHER_E5M2 || mode == FEATHER_E4M3, FEATHER_EMODE,
                   "feather_flash_attn_fp8: mode %d not supported", mode);
+    FEATHER_CHECK(workspace_bytes >= 0 && (workspace || workspace_bytes == 0) && aligned(workspace, 16), FEATHER_EINVAL,
+                  "feather_flash_attn_fp8_ws: workspace must be 16-byte aligned, its size not negative");
     FEATHER_CHECK(tail == FEATHER_TAIL_MASK || tail == FEATHER_TAIL_REFERENCE, FEATHER_EINVAL,
                   "feather_flash_attn_fp8: bad tail flag %d", tail);
     FEATHER_CHECK(n_heads >= 0 && L >= 0 && d > 0, FEATHER_EINVAL, "feather_flash_attn_fp8: negative shape");
@@ -960,7 +1086,8 @@ extern "C" int feather_flash_attn_fp8(const void *q, const void *k, const void *
     FEATHER_CHECK(aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out_f32, 16), FEATHER_EINVAL,
                   "feather_flash_attn_fp8: pointers must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
-    const AttnArgs a = {q, k, v, out_f32, n_heads, L, kv_group, scale, tail, nullptr, 0, 0, 0, 0};
+    const AttnArgs a = {q, k, v, out_f32, n_heads, L, kv_group, scale, tail, nullptr, 0, 0, 0, 0, workspace,
+                        workspace_bytes};
     if (mode == FEATHER_E5M2) return dispatch_attn<FEATHER_E5M2, false>(a, d, s);
     return dispatch_attn<FEATHER_E4M3, false>(a, d, s);
 }
@@ -988,7 +1115,7 @@ extern "C" int feather_flash_attn_fp8_varlen(const void *q, const void *k, const
                   FEATHER_EINVAL, "%s: q/k/v/out must be 16-byte aligned", me);
     hipStream_t s = (hipStream_t)stream;
     const AttnArgs a = {q, k, v, out_f32, n_heads, 0, kv_group, scale, FEATHER_TAIL_MASK, cu_seqlens, n_seq,
-                        max_seqlen, total_rows, causal};
+                        max_seqlen, total_rows, causal, nullptr, 0};
     if (mode == FEATHER_E5M2) return dispatch_attn<FEATHER_E5M2, true>(a, d, s);
     return dispatch_attn<FEATHER_E4M3, true>(a, d, s);
 }

@@ -262,6 +262,28 @@ __device__ __forceinline__ float max_xor32(float x) {
     return a;
 }
 
+// Results of the matrix core are not interlocked against the vector ALU: a vector instruction that reads an MFMA
+// result needs 7 / 11 / 19 cycles of distance from a 4- / 8- / 16-pass MFMA.  The compiler counts these wait states
+// for the instructions it emits itself, but it does not look into asm statements, so an asm statement must never be
+// the first reader of an MFMA result: max3_raw on fresh scores now and then took the maximum over accumulators that
+// the last MFMA of the chain had not updated yet -- harmless for the result (the reference point of the softmax may
+// be any value), but different from run to run.  mfma_settle takes the N accumulators at `acc` as operands, which
+// places it after the MFMAs that write them and before every later reader, and lets 12 cycles pass (MFMAs retire in
+// order, so the distance to the last one covers all).  For 4- and 8-pass MFMAs.
+#define FEATHER_SETTLE_NOPS "s_nop 7\n\ts_nop 3"
+template <int N>
+__device__ __forceinline__ void mfma_settle(float4_t *a) {
+    static_assert(N == 1 || N == 2 || N == 4 || N == 8 || N == 16, "accumulator count");
+    if constexpr (N == 1) asm volatile(FEATHER_SETTLE_NOPS : "+v"(a[0]));
+    if constexpr (N == 2) asm volatile(FEATHER_SETTLE_NOPS : "+v"(a[0]), "+v"(a[1]));
+    if constexpr (N == 4) asm volatile(FEATHER_SETTLE_NOPS : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]));
+    if constexpr (N == 8)
+        asm volatile(FEATHER_SETTLE_NOPS : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
+    if constexpr (N == 16)
+        asm volatile(FEATHER_SETTLE_NOPS : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
+                     "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
+}
+
 // max of two / three floats as single instructions.  In front of fmaxf the compiler puts a canonicalising
 // max(x, x) on every value whose NaN quietness it cannot prove (MFMA results, values that came out of
 // inline asm): 4 of the ~80 vector instructions of a softmax block.  Scores are never signalling

@@ -324,6 +324,7 @@ __global__ __launch_bounds__(kPaThreads) void paged_attn_split_kernel(
                 s[a] = pa_mfma16(pa_dec8<MODE>(S.kw[a][c64].z, S.kw[a][c64].w), qf[2 * c64 + 1], s[a]);
             }
         }
+        mfma_settle<2>(s);   // the first readers of the scores are asm statements (max3_raw)
         // online softmax (lane column = query head), log2 domain; only the last step of a split
         // can hold tokens past its end (wave-uniform test)
         if (t0 + kStepTok > t_end) {

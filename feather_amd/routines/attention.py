@@ -23,9 +23,10 @@ _TAILS = {"mask": N.TAIL_MASK, "reference": N.TAIL_REFERENCE}
 
 def flash_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seq_len: int, h_dim: int, *,
                                      mode: str = "E5M2", scale: float | None = None, tail: str = "mask",
-                                     kv_group: int = 1, causal: bool = False) -> torch.Tensor:
+                                     kv_group: int = 1, causal: bool = False, workspace: bool = True) -> torch.Tensor:
     """``softmax(Q K^T * scale) V`` per head; non-causal unless ``causal=True``
-    (query ``i`` then sees keys ``0..i``; needs ``tail="mask"``).
+    (query ``i`` then sees keys ``0..i``; needs ``tail="mask"``).  ``workspace=False`` keeps the call from
+    allocating the scratch tensor that short sequences of few wide heads use to spread over the whole GPU.
 
     ``q`` holds ``n_heads * seq_len * h_dim`` packed words (``h_dim = d // 4``);
     ``k``/``v`` hold ``n_heads // kv_group`` heads.  Returns float32
@@ -65,7 +66,10 @@ def flash_attention_fp8_acc_fp32_gpu(q: torch.Tensor, k: torch.Tensor, v: torch.
         cu = torch.arange(2, dtype=torch.int32, device=q.device) * seq_len   # [0, L], built on the device (graph-capturable)
         N.call(q.device, "feather_flash_attn_fp8_varlen", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(cu), 1, seq_len, seq_len, n_heads, d, kv_group, code, float(scale), 1)
     else:
-        N.call(q.device, "feather_flash_attn_fp8", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), n_heads, seq_len, d, kv_group, code, float(scale), _TAILS[tail])
+        # few short wide heads: the library cuts the key loop over more workgroups if it is given room for the partial results
+        ws_bytes = int(N.lib().feather_flash_attn_workspace_bytes(n_heads, seq_len, d)) if workspace else 0
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+        N.call(q.device, "feather_flash_attn_fp8_ws", N.ptr(q), N.ptr(k), N.ptr(v), N.ptr(out), N.ptr(ws) if ws_bytes else None, ws_bytes, n_heads, seq_len, d, kv_group, code, float(scale), _TAILS[tail])
     if q.dim() >= 2 and q.shape[-2:] == (seq_len, h_dim):
         return out.view(*q.shape[:-2], seq_len, d)
     return out[0] if n_heads == 1 else out

@@ -55,7 +55,7 @@ extern "C" {
 /* Library version (major * 10000 + minor * 100 + patch); FEATHER_HIP_VERSION is the version of this header.
  * A change of any signature or struct below raises the minor number: a binding must refuse a library whose
  * feather_version() differs from the header it was written against in major or minor. */
-#define FEATHER_HIP_VERSION 10300
+#define FEATHER_HIP_VERSION 10400
 int feather_version(void);
 
 /* Message for the last non-zero return code on this thread ("" if none). */
@@ -145,6 +145,18 @@ int feather_dot_fp16(const void *x1, const void *x2, void *out_f32, void *scratc
  * scale = 1/sqrt(d), tail = REFERENCE. */
 int feather_flash_attn_fp8(const void *q, const void *k, const void *v, void *out_f32, int64_t n_heads, int64_t L,
                            int64_t d, int64_t kv_group, int mode, float scale, int tail, void *stream);
+
+/* The same attention with an optional device workspace.  Short sequences of few wide heads make a grid that leaves
+ * most of the 256 CUs idle (8 heads x 1024 rows at d = 512: 128 workgroups); with a workspace of
+ * feather_flash_attn_workspace_bytes(n_heads, L, d) bytes (0: the shape does not profit) the key loop of every query
+ * tile is cut into 2 or 4 ranges that run as separate workgroups and a second small kernel combines them (same
+ * result to the rounding of the fp32 additions).  workspace == NULL, or a workspace smaller than asked for, runs
+ * fewer ranges or the plain kernel; nothing is kept in the workspace between calls.  No reference counterpart
+ * (the reference launches one program per 64 queries of one head, attention.py:172-179). */
+int64_t feather_flash_attn_workspace_bytes(int64_t n_heads, int64_t L, int64_t d);
+int feather_flash_attn_fp8_ws(const void *q, const void *k, const void *v, void *out_f32, void *workspace,
+                              int64_t workspace_bytes, int64_t n_heads, int64_t L, int64_t d, int64_t kv_group, int mode,
+                              float scale, int tail, void *stream);
 
 /* Attention forward on packed variable-length sequences, optionally causal.  No reference
  * counterpart (the reference kernel, feather/routines/attention.py:14-108, is one

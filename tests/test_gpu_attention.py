@@ -60,6 +60,69 @@ def test_flash_attention_vs_oracle(dev, orc, mode, heads, L, d):
         assert _nerr(got, orc.flash_attn(q, k, v, L, d, mode)) <= TOL
 
 
+@pytest.mark.parametrize("mode,heads,L,d,tail,ranges", [
+    ("E4M3", 2, 512, 256, "mask", 2), ("E5M2", 1, 1000, 256, "mask", 4), ("E4M3", 1, 1000, 256, "reference", 4),
+    ("E4M3", 1, 300, 512, "mask", 2), ("E5M2", 2, 530, 512, "mask", 4), ("E4M3", 1, 530, 512, "reference", 4),
+    ("E5M2", 2, 1100, 128, "mask", 4), ("E4M3", 3, 600, 128, "mask", 2), ("E4M3", 8, 1024, 512, "mask", 2),
+])
+def test_flash_attention_key_ranges_over_workgroups(dev, orc, mode, heads, L, d, tail, ranges):
+    """Few short wide heads: with a workspace the key loop of every query tile is cut into `ranges` ranges that
+    run as separate workgroups and are combined by a second kernel.  Same result as the oracle, and as the plain
+    kernel up to the rounding of P (the ranges have other reference points) and of the fp32 additions; ragged last
+    ranges (17 tiles in ranges of 5), both tail modes, and what a missing or short workspace does."""
+    from feather_amd import _native as N
+    from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
+    lib = N.lib()
+    need = int(lib.feather_flash_attn_workspace_bytes(heads, L, d))
+    assert need == ranges * heads * L * (d + 2) * 4
+    rng = np.random.default_rng(heads * 1000 + L + d)
+    q, k, v = _qkv(rng, heads, L, d, mode, orc)
+    qd, kd, vd = (_dev_words(t, dev) for t in (q, k, v))
+    got = flash_attention_fp8_acc_fp32_gpu(qd, kd, vd, L, d // 4, mode=mode, tail=tail).cpu().numpy().reshape(heads, L, d)
+    plain = flash_attention_fp8_acc_fp32_gpu(qd, kd, vd, L, d // 4, mode=mode, tail=tail, workspace=False)
+    plain = plain.cpu().numpy().reshape(heads, L, d)
+    if tail == "mask":
+        assert _nerr(got, orc.attention_f64_np(q, k, v, L, d, mode)) <= TOL
+    else:
+        assert _nerr(got, orc.flash_attn(q, k, v, L, d, mode, tail_reference=True)) <= TOL
+    assert _nerr(got, plain) <= 5e-4
+    assert not np.array_equal(got, plain)          # the ranges did run
+    # through the C ABI: a workspace too small for two ranges runs the plain kernel (bit-identical), one that holds
+    # half of what was asked for runs half the ranges
+    code, scale = N.mode_code(mode), 1.0 / float(np.sqrt(d))      # the wrapper's default, to the bit
+    tl = N.TAIL_MASK if tail == "mask" else N.TAIL_REFERENCE
+    for ws_bytes, same_as_plain in ((2 * heads * L * (d + 2) * 4 - 16, True), (need // 2, ranges == 2), (need, False)):
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        out = torch.full((heads, L, d), float("nan"), dtype=torch.float32, device=dev)
+        N.check(lib.feather_flash_attn_fp8_ws(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), ws.data_ptr(),
+                                              ws_bytes, heads, L, d, 1, code, scale, tl, N.stream_ptr(dev)))
+        torch.cuda.synchronize()
+        o = out.cpu().numpy()
+        assert np.isfinite(o).all()
+        assert np.array_equal(o, plain) == same_as_plain
+        assert _nerr(o, plain) <= 5e-4
+
+
+@pytest.mark.parametrize("mode", ["E4M3", "E5M2"])
+@pytest.mark.parametrize("heads,L,d", [(8, 1024, 512), (1, 300, 512), (2, 530, 512), (8, 1024, 256), (8, 1024, 128),
+                                         (8, 2048, 64), (4, 600, 32)])
+def test_flash_attention_is_identical_from_call_to_call(dev, mode, heads, L, d):
+    """Six calls on the same operands give the same bits.  (An asm statement that was the first reader of the score
+    MFMA's result did not get the wait states the compiler inserts for its own instructions, and in the shape with 16
+    keys per wave group -- d = 512 below 256 workgroups -- the row maximum was now and then taken from accumulators
+    that the last MFMA had not updated yet: a valid result with another reference point, but another one from call to
+    call.)  With and without the workspace for key ranges."""
+    from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
+    import feather_amd as feather
+    g = torch.Generator(device=dev).manual_seed(heads + L + d)
+    q, k, v = (feather.pack_fp8_tensor(torch.randn(heads, L, d, generator=g, device=dev).half(), mode=mode).view(heads, L, d // 4)
+               for _ in range(3))
+    for ws in (False, True):
+        first = flash_attention_fp8_acc_fp32_gpu(q, k, v, L, d // 4, mode=mode, workspace=ws)
+        for _ in range(5):
+            assert torch.equal(flash_attention_fp8_acc_fp32_gpu(q, k, v, L, d // 4, mode=mode, workspace=ws), first)
+
+
 def test_flash_attention_reference_signature_and_ints(dev, orc):
     """Reference call shape: 2-D [L, d/4] words, h_dim = d // 4, E5M2, integer inputs as in
     bench_attention.py:52-59, output [L, d] fp32 in the original column order."""

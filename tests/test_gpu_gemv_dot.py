@@ -102,11 +102,13 @@ def test_gemv_e4m3_uses_kernel_decode_not_ieee(dev, orc):
         assert _nerr(out, want) <= 1e-4
 
 
-def test_gemv_config_sized_properties(dev):
+def test_gemv_config_sized_properties(dev, orc):
     """16384 x 16384 (too large for the scalar oracle): linearity in the vector and agreement
     with a torch float64 matvec of the operands decoded by the HIP unpack kernel, both on device.  That
-    check leans on the unpack kernel, which test_gpu_pack.py holds bit-exact to the oracle's decode on
-    all 256 codes of both modes in the same run."""
+    check leans on the unpack kernel (which test_gpu_pack.py holds bit-exact to the oracle's decode on
+    all 256 codes of both modes in the same run), so 1 024 rows -- the first and last rows of the matrix, of
+    eight-row groups and of random positions -- are also checked without it: their packed words are copied to
+    the host, decoded by the oracle's table and summed in float64."""
     import feather_amd as feather
     g = torch.Generator().manual_seed(2)
     M = K = 16384
@@ -121,6 +123,15 @@ def test_gemv_config_sized_properties(dev):
         vd = feather.unpack_fp8_tensor(vp, mode=mode, semantics="kernel")
         want = torch.mv(md.double(), vd.double())
         assert ((out.double() - want).abs().max() / want.abs().max()).item() <= 1e-4
+        rows = np.unique(np.concatenate([np.arange(16), M - 1 - np.arange(16), 8 * np.arange(0, M // 8, 37),
+                                         8 * np.arange(0, M // 8, 41) + 7,
+                                         np.random.default_rng(3).integers(0, M, 400)]))
+        words = mp.view(torch.int32).view(M, K // 4)[torch.from_numpy(rows).to(dev)].cpu().numpy().view(np.uint32)
+        m_host = orc.decode_np(words.reshape(-1), mode).reshape(len(rows), K).astype(np.float64)
+        v_host = orc.decode_np(vp.view(torch.int32).cpu().numpy().view(np.uint32), mode)[:K].astype(np.float64)
+        want_rows = m_host @ v_host
+        got_rows = out.cpu().numpy().astype(np.float64)[rows]
+        assert np.abs(got_rows - want_rows).max() / np.abs(want_rows).max() <= 1e-4
         # twice the vector (exact in FP8: exponent + 1) doubles the result exactly
         vp2 = feather.pack_fp8_tensor((2 * v.half()).to(dev), mode=mode)
         vd2 = feather.unpack_fp8_tensor(vp2, mode=mode, semantics="kernel")

@@ -95,6 +95,15 @@ def test_c_abi_argument_checks_without_gpu():
                                     0.1, None) == N.ESHAPE                           # paged decode: 64, 128, 256, 512
     assert L.feather_paged_cache_write(None, None, 0, None, None, None, None, None, 1, 4, 2, 64, 16, 4, -1, N.E5M2,
                                        None) == N.EINVAL
+    # attention with a workspace: how much the library asks for (pure host arithmetic) and its argument checks
+    ws = L.feather_flash_attn_workspace_bytes
+    assert ws(8, 1024, 512) == 2 * 8 * 1024 * 514 * 4      # 128 workgroups: two key ranges fill the 256 CUs
+    assert ws(8, 1024, 128) == 4 * 8 * 1024 * 130 * 4      # 64 workgroups of 128 queries: four ranges
+    assert ws(8, 4096, 512) == 0 and ws(64, 8192, 64) == 0 and ws(1, 100, 256) == 0 and ws(0, 64, 256) == 0
+    assert L.feather_flash_attn_fp8_ws(None, None, None, None, 8, 64, 1, 64, 64, 1, N.E5M2, 0.1, 0, None) == N.EINVAL
+    assert b"workspace" in L.feather_last_error()          # misaligned
+    assert L.feather_flash_attn_fp8_ws(None, None, None, None, None, 64, 1, 64, 64, 1, N.E5M2, 0.1, 0, None) == N.EINVAL
+    assert L.feather_flash_attn_fp8_ws(None, None, None, None, None, 0, 0, 64, 64, 1, N.E5M2, 0.1, 0, None) == N.OK
 
 
 def test_error_mapping():

@@ -436,6 +436,10 @@ def main() -> int:
             us_sdpa = gpu_time_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 10, 10, sync, warm_ms)
             extra[f"sdpa_fp16_b1h8_d{d}_L{L}_us"] = round(us_sdpa, 1)
             arl[key] = mfma_record(busy, key, f"flash_attn_kernel<{d}, E4M3>", 4.0 * B * H * L * L * d, us, 0.0, us_sdpa)
+            ws_bytes = int(N.lib().feather_flash_attn_workspace_bytes(B * H, L, d))
+            if ws_bytes:   # a grid below 256 workgroups: key ranges over workgroups + a merge kernel (the wrapper's default)
+                arl[key]["key_ranges"] = ws_bytes // (B * H * L * (d + 2) * 4)
+                arl[key]["workspace_bytes"] = ws_bytes
             del qkv16, pk
         torch.cuda.empty_cache()
         # paged-attention decode, 32 sequences x 32 query heads over 4 KV heads, d=64, E4M3, blocks of 16

@@ -441,6 +441,26 @@ def main() -> int:
                 arl[key]["key_ranges"] = ws_bytes // (B * H * L * (d + 2) * 4)
                 arl[key]["workspace_bytes"] = ws_bytes
             del qkv16, pk
+        # the reference harness's own grid (benchmark/bench_attention.py:13-14): ONE head of 128 .. 8192 rows at head
+        # dims 64 / 256 / 512, E5M2, the reference-named entry point with its tail semantics.  A single head makes 2 to
+        # 128 workgroups; the wrapper hands the library a workspace and the key loop is cut into ranges over more
+        # workgroups.  Device time by graph replay for both sides (the short ones are below the host's per-call cost).
+        for d in (64, 256, 512):
+            for L in (128, 256, 512, 1024, 4096, 8192):
+                qkv16 = [randn(1, 1, L, d).half() for _ in range(3)]
+                pk = [feather.pack_fp8_tensor(t[0, 0], mode="E5M2").view(L, d // 4) for t in qkv16]
+                us = gpu_time_graph_us(lambda i: feather.flash_attention_fp8_e5m2_acc_fp32_gpu(pk[0], pk[1], pk[2], L, d // 4),
+                                       16, sync)
+                us_sdpa = gpu_time_graph_us(lambda i: torch.nn.functional.scaled_dot_product_attention(*qkv16), 16, sync)
+                key = f"flash_attn_e5m2_h1_d{d}_L{L}"
+                extra[key + "_us"] = round(us, 2)
+                extra[f"sdpa_fp16_h1_d{d}_L{L}_us"] = round(us_sdpa, 2)
+                kern = "flash_attn64_wide_kernel<E5M2>" if d == 64 else f"flash_attn_kernel<{d}, E5M2>"
+                arl[key] = mfma_record(busy, key, kern, 4.0 * L * L * d, us, 0.5, us_sdpa)
+                arl[key]["timing"] = "graph"
+                ws_bytes = int(N.lib().feather_flash_attn_workspace_bytes(1, L, d))
+                arl[key]["key_ranges"] = ws_bytes // (L * (d + 2) * 4) if ws_bytes else 1
+                del qkv16, pk
         torch.cuda.empty_cache()
         # paged-attention decode, 32 sequences x 32 query heads over 4 KV heads, d=64, E4M3, blocks of 16
         # tokens scattered by a random block table; bytes = K and V codes of every context token once
@@ -487,9 +507,10 @@ def main() -> int:
                 for name in ("k_cache", "v_cache"):
                     vals = randn(nb_ * cfg.n_kv_heads * bs * cfg.head_dim).half()
                     lay[name].view(-1).copy_(feather.pack_fp8_tensor(vals, mode=mode).view(torch.int32))
-            btd = torch.randperm(nb_, generator=g, device=dev).to(torch.int32).view(batch, cmax // bs)
-            cl = torch.randint(512, cmax, (batch,), generator=g, device=dev, dtype=torch.int32)
-            tok = torch.randint(0, cfg.vocab, (batch,), generator=g, device=dev, dtype=torch.int32)
+            gd = torch.Generator(device=dev).manual_seed(100 + batch)   # the step's own draw: the same contexts in every run
+            btd = torch.randperm(nb_, generator=gd, device=dev).to(torch.int32).view(batch, cmax // bs)
+            cl = torch.randint(512, cmax, (batch,), generator=gd, device=dev, dtype=torch.int32)
+            tok = torch.randint(0, cfg.vocab, (batch,), generator=gd, device=dev, dtype=torch.int32)
             logits = torch.empty((batch, cfg.vocab), dtype=torch.float32, device=dev)
             us = gpu_time_us(lambda i: dec.step(tok, btd, cl, out=logits), 20, 10, sync, warm_ms)
             step_bytes = dec.weight_bytes() + int(cl.sum().item()) * 2 * cfg.n_kv_heads * cfg.head_dim * cfg.n_layers

@@ -514,38 +514,38 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn_kernel(
     }
 }
 
-// Combines the key ranges of flash_attn_kernel<..., ZS = true>: one thread per (row, four dims).  Range z of a row
+constexpr int kMaxKeyChunks = 8;
+
+// Combines the Z key ranges of flash_attn_kernel<..., ZS = true> and flash_attn64_wide_kernel<..., ZS = true>:
+// one thread per (row, four dims).  Range z of a row
 // holds O_z = sum_k 2^((s_k - m_z) c) V_k and l_z = sum_k 2^((s_k - m_z) c); with m = max_z m_z the row is
 // sum_z 2^((m_z - m) c) O_z / sum_z 2^((m_z - m) c) l_z, added in range order.
+template <int Z>
 __global__ __launch_bounds__(256) void flash_attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out,
-                                                               int64_t rows_total, int dq, int n_kchunks,
-                                                               float scale_log2e) {
+                                                               int64_t rows_total, int dq, float scale_log2e) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= rows_total * dq) return;
     const int64_t row = idx / dq;
-    const float2v_t *ml = reinterpret_cast<const float2v_t *>(part + (int64_t)n_kchunks * rows_total * dq * 4);
+    const float2v_t *ml = reinterpret_cast<const float2v_t *>(part + (int64_t)Z * rows_total * dq * 4);
     const float4_t *po = reinterpret_cast<const float4_t *>(part);
-    float2v_t mlz[4];
-    float4_t oz[4];
+    float2v_t mlz[Z];
+    float4_t oz[Z];
 #pragma unroll
-    for (int z = 0; z < 4; z++)
-        if (z < n_kchunks) {
-            mlz[z] = ml[z * rows_total + row];
-            oz[z] = po[z * rows_total * dq + idx];
-        }
+    for (int z = 0; z < Z; z++) {   // every load goes out before the first use
+        mlz[z] = ml[z * rows_total + row];
+        oz[z] = __builtin_nontemporal_load(po + z * rows_total * dq + idx);
+    }
     float m = mlz[0][0];
 #pragma unroll
-    for (int z = 1; z < 4; z++)
-        if (z < n_kchunks) m = fmaxf(m, mlz[z][0]);
+    for (int z = 1; z < Z; z++) m = fmaxf(m, mlz[z][0]);
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
     float l = 0.f;
 #pragma unroll
-    for (int z = 0; z < 4; z++)
-        if (z < n_kchunks) {
-            const float w = mlz[z][0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mlz[z][0] - m) * scale_log2e);
-            acc += oz[z] * w;
-            l += mlz[z][1] * w;
-        }
+    for (int z = 0; z < Z; z++) {
+        const float w = mlz[z][0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mlz[z][0] - m) * scale_log2e);
+        acc += oz[z] * w;
+        l += mlz[z][1] * w;
+    }
     reinterpret_cast<float4_t *>(out)[idx] = acc / l;
 }
 
@@ -572,12 +572,13 @@ __global__ __launch_bounds__(256) void flash_attn_merge_kernel(const float *__re
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef int int8v_t __attribute__((ext_vector_type(8)));
 
-template <int MODE, bool VC, int WAVES, int OCC>
+template <int MODE, bool VC, int WAVES, int OCC, bool ZS = false>
 __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
     const uint32_t *__restrict__ q, const uint32_t *__restrict__ k, const uint32_t *__restrict__ v,
     float *__restrict__ out, int L, int n_heads, int kv_group, int tiles_per_head, float scale_log2e,
     int keys_scored, int mask_tail, const int32_t *__restrict__ cu_seqlens, int tiles_per_seq, int total_rows,
-    int causal) {
+    int causal, float *__restrict__ part, int kchunk_keys, int n_kchunks) {
+    static_assert(!(ZS && VC), "key ranges over workgroups are for fixed-length heads");
     constexpr int D = 64, DW = 16, BN = 64;
     constexpr bool BF8 = MODE == FEATHER_E5M2;   // K and Q stay packed bytes; otherwise both are decoded to fp16
     constexpr int KP = (BF8 ? D : 2 * D) + 16;   // K row pitch in LDS, bytes
@@ -596,6 +597,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
     int bid = blockIdx.x;
     const int total = gridDim.x;
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;   // an XCD works through contiguous (head, tile) pairs
+    int zchunk = 0;
+    if constexpr (ZS) {   // key ranges of a query tile (see flash_attn_kernel): neighbours in this order
+        zchunk = bid % n_kchunks;
+        bid /= n_kchunks;
+    }
     const int head = bid / tiles_per_head;
     int tile = bid % tiles_per_head;
     const int kv_head = head / kv_group;
@@ -738,9 +744,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
         }
     };
 
-    prefetch(0);
+    const int key_begin = ZS ? zchunk * kchunk_keys : 0;
+    const int key_end = ZS ? min(keys_scored, key_begin + kchunk_keys) : keys_scored;
+    prefetch(key_begin);
     stage(0);
-    if (BN < keys_scored) prefetch(BN);
+    if (key_begin + BN < key_end) prefetch(key_begin + BN);
     __syncthreads();
     // One key tile; the buffer index is a compile-time constant (the loop below is unrolled by two), so every
     // LDS address is a loop-invariant per-lane register plus an immediate offset instead of vector adds per tile.
@@ -755,8 +763,8 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
             skip = causal && key0 > q0 + 63;              // every key lies past the wave's last query
         }
         if constexpr (VC) {   // a wave with nothing to score in this tile still stages: one copy of that code, up front
-            if (key0 + BN < keys_scored) stage(cur ^ 1);
-            if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);
+            if (key0 + BN < key_end) stage(cur ^ 1);
+            if (key0 + 2 * BN < key_end) prefetch(key0 + 2 * BN);
         }
         if (!skip) {
             // ---- S^T = K Q^T, raw scores: [query block][key block]
@@ -778,7 +786,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
                     vf[g][d] = *reinterpret_cast<const half8_t *>(vt_lds + row * VS + (((2 * g + h) ^ swz(row)) << 3));
                 }
             // the next tile goes to the other buffer while this tile's fragments are on their way from LDS
-            if constexpr (!VC) if (key0 + BN < keys_scored) stage(cur ^ 1);
+            if constexpr (!VC) if (key0 + BN < key_end) stage(cur ^ 1);
             float16_t sc[2][2];
             const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             if constexpr (BF8) {
@@ -801,7 +809,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
                             sc[b][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(k16[st], qh16[b][st], st == 0 ? zero16 : sc[b][c], 0, 0, 0);
                 }
             }
-            if constexpr (!VC) if (key0 + 2 * BN < keys_scored) prefetch(key0 + 2 * BN);   // the tile after that into registers
+            if constexpr (!VC) if (key0 + 2 * BN < key_end) prefetch(key0 + 2 * BN);   // the tile after that into registers
 #pragma unroll
             for (int b = 0; b < 2; b++) {
                 // ---- online softmax of one 32-query block; p = 2^(s * c - m * c) on the raw-score maximum
@@ -870,18 +878,24 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void flash_attn64_wide_kernel(
         }
         __syncthreads();  // tile i+1 is visible; every wave is done reading tile i
     };
-    for (int key0 = 0; key0 < keys_scored; key0 += 2 * BN) {
+    for (int key0 = key_begin; key0 < key_end; key0 += 2 * BN) {
         tile_body(key0, std::integral_constant<int, 0>{});
-        if (key0 + BN < keys_scored) tile_body(key0 + BN, std::integral_constant<int, 1>{});
+        if (key0 + BN < key_end) tile_body(key0 + BN, std::integral_constant<int, 1>{});
     }
 
     // ---- epilogue: the two lanes of a query add their shares of the row sum; normalise, store [q][dd]
-    float *oh = out + q_row0 * D;
+    // (a key range: unnormalised, with the reference point and the row sum beside it)
+    const int64_t rows_total = (int64_t)n_heads * L;
+    float *oh = ZS ? part + ((int64_t)zchunk * rows_total + q_row0) * D : out + q_row0 * D;
 #pragma unroll
     for (int b = 0; b < 2; b++) {
         const float other = as_float((uint32_t)__builtin_amdgcn_ds_bpermute(4 * (lane ^ 32), (int)as_u32(l_run[b])));
-        const float l = l_run[b] + other;
+        const float l = ZS ? 1.f : l_run[b] + other;
         const int row = q0 + 32 * b + n;
+        if constexpr (ZS)
+            if (row < L && h == 0)
+                *reinterpret_cast<float2v_t *>(part + (int64_t)n_kchunks * rows_total * D +
+                                               ((int64_t)zchunk * rows_total + q_row0 + row) * 2) = float2v_t{m_run[b], l_run[b] + other};
         if (row < L) {
 #pragma unroll
             for (int d = 0; d < 2; d++)
@@ -909,10 +923,38 @@ struct AttnArgs {
     int64_t ws_bytes;
 };
 
-constexpr int kMaxKeyChunks = 4;
 // Bytes of workspace that n_kchunks key ranges of n_heads * L rows need: accumulators, then (m, l) pairs.
 static int64_t key_chunk_ws_bytes(int64_t n_heads, int64_t L, int64_t d, int n_kchunks) {
     return n_kchunks * n_heads * L * (d + 2) * 4;
+}
+
+// Key ranges of whole BN-key tiles, every range starting below the last scored key: keys per range, and the number
+// of ranges that leaves.
+static void key_range_plan(int64_t keys_scored, int bn, int &n_kchunks, int64_t &kchunk_keys) {
+    const int64_t n_tiles_k = keys_scored / bn;
+    kchunk_keys = (n_tiles_k + n_kchunks - 1) / n_kchunks * bn;
+    n_kchunks = (int)((keys_scored + kchunk_keys - 1) / kchunk_keys);
+}
+
+static int launch_key_range_merge(const AttnArgs &a, int d, int n_kchunks, hipStream_t s) {
+    const int64_t rows_total = a.n_heads * a.L, quads = rows_total * (d / 4);
+    const dim3 grid((unsigned)((quads + 255) / 256)), block(256);
+    const float c = a.scale * 1.4426950408889634f;
+    const float *part = (const float *)a.ws;
+    float *out = (float *)a.out;
+    switch (n_kchunks) {
+        case 2: hipLaunchKernelGGL(flash_attn_merge_kernel<2>, grid, block, 0, s, part, out, rows_total, d / 4, c); break;
+        case 3: hipLaunchKernelGGL(flash_attn_merge_kernel<3>, grid, block, 0, s, part, out, rows_total, d / 4, c); break;
+        case 4: hipLaunchKernelGGL(flash_attn_merge_kernel<4>, grid, block, 0, s, part, out, rows_total, d / 4, c); break;
+        case 5: hipLaunchKernelGGL(flash_attn_merge_kernel<5>, grid, block, 0, s, part, out, rows_total, d / 4, c); break;
+        case 6: hipLaunchKernelGGL(flash_attn_merge_kernel<6>, grid, block, 0, s, part, out, rows_total, d / 4, c); break;
+        case 7: hipLaunchKernelGGL(flash_attn_merge_kernel<7>, grid, block, 0, s, part, out, rows_total, d / 4, c); break;
+        case 8: hipLaunchKernelGGL(flash_attn_merge_kernel<8>, grid, block, 0, s, part, out, rows_total, d / 4, c); break;
+        default:
+            set_error("feather_flash_attn_fp8: %d key ranges", n_kchunks);
+            return FEATHER_EINVAL;
+    }
+    return check_launch("feather_flash_attn_fp8 (merge of the key ranges)");
 }
 
 template <int D, int MODE, int QB, int SB, int BN, int OCC, bool VC, int WAVES = 4, int KSPLIT = 1, bool ZS = false>
@@ -929,10 +971,8 @@ static int launch_attn(const AttnArgs &a, hipStream_t s, int n_kchunks = 1) {
     // the reference scores whole 64-key tiles (zero rows past L); otherwise only tiles of BN up to L
     int64_t keys_scored = a.tail == FEATHER_TAIL_REFERENCE ? (L + 63) / 64 * 64 : (L + BN - 1) / BN * BN;
     auto kern = flash_attn_kernel<D, MODE, QB, SB, BN, OCC, VC, WAVES, KSPLIT, ZS>;
-    // key ranges: whole tiles, every range starting below the last scored key
-    const int64_t n_tiles_k = keys_scored / BN;
-    const int64_t kchunk_keys = (n_tiles_k + n_kchunks - 1) / n_kchunks * BN;
-    if (ZS) n_kchunks = (int)((keys_scored + kchunk_keys - 1) / kchunk_keys);
+    int64_t kchunk_keys = keys_scored;
+    if (ZS) key_range_plan(keys_scored, BN, n_kchunks, kchunk_keys);
     static unsigned long long lds_raised = 0;   // per instantiation, one bit per device
     hipError_t e = raise_lds_limit(reinterpret_cast<const void *>(kern), lds, lds_raised);
     FEATHER_CHECK(e == hipSuccess, FEATHER_ELAUNCH, "feather_flash_attn_fp8: cannot raise LDS limit: %s",
@@ -945,14 +985,11 @@ static int launch_attn(const AttnArgs &a, hipStream_t s, int n_kchunks = 1) {
                        (int)a.total_rows, a.causal, (float *)a.ws, (int)kchunk_keys, n_kchunks);
     int rc = check_launch("feather_flash_attn_fp8");
     if (!ZS || rc != FEATHER_OK) return rc;
-    const int64_t rows_total = a.n_heads * L, quads = rows_total * (D / 4);
-    hipLaunchKernelGGL(flash_attn_merge_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s,
-                       (const float *)a.ws, (float *)a.out, rows_total, D / 4, n_kchunks, a.scale * log2e);
-    return check_launch("feather_flash_attn_fp8 (merge of the key ranges)");
+    return launch_key_range_merge(a, D, n_kchunks, s);
 }
 
-template <int MODE, bool VC, int WAVES, int OCC>
-static int launch_attn64_wide(const AttnArgs &a, hipStream_t s) {
+template <int MODE, bool VC, int WAVES, int OCC, bool ZS = false>
+static int launch_attn64_wide(const AttnArgs &a, hipStream_t s, int n_kchunks = 1) {
     constexpr int QT = 64 * WAVES, BN = 64, D = 64;
     constexpr size_t lds = (size_t)(BN * ((MODE == FEATHER_E5M2 ? D : 2 * D) + 16) + D * BN * 2) * 2;   // two (K, V^T fp16) buffers
     const int64_t L = VC ? a.max_seqlen : a.L;
@@ -964,12 +1001,16 @@ static int launch_attn64_wide(const AttnArgs &a, hipStream_t s) {
     // both tail modes score whole 64-key tiles here (the reference scores zero rows past L, the mask hides them)
     const int64_t keys_scored = (L + BN - 1) / BN * BN;
     const float log2e = 1.4426950408889634f;
-    hipLaunchKernelGGL((flash_attn64_wide_kernel<MODE, VC, WAVES, OCC>), dim3((unsigned)blocks), dim3(64 * WAVES), lds, s,
-                       (const uint32_t *)a.q, (const uint32_t *)a.k, (const uint32_t *)a.v, (float *)a.out, (int)L,
-                       (int)a.n_heads, (int)a.kv_group, (int)tiles, a.scale * log2e, (int)keys_scored,
-                       a.tail == FEATHER_TAIL_MASK ? 1 : 0, (const int32_t *)a.cu_seqlens, tiles_per_seq,
-                       (int)a.total_rows, a.causal);
-    return check_launch("feather_flash_attn_fp8");
+    int64_t kchunk_keys = keys_scored;
+    if (ZS) key_range_plan(keys_scored, BN, n_kchunks, kchunk_keys);
+    hipLaunchKernelGGL((flash_attn64_wide_kernel<MODE, VC, WAVES, OCC, ZS>), dim3((unsigned)(blocks * (ZS ? n_kchunks : 1))),
+                       dim3(64 * WAVES), lds, s, (const uint32_t *)a.q, (const uint32_t *)a.k, (const uint32_t *)a.v,
+                       (float *)a.out, (int)L, (int)a.n_heads, (int)a.kv_group, (int)tiles, a.scale * log2e,
+                       (int)keys_scored, a.tail == FEATHER_TAIL_MASK ? 1 : 0, (const int32_t *)a.cu_seqlens, tiles_per_seq,
+                       (int)a.total_rows, a.causal, (float *)a.ws, (int)kchunk_keys, n_kchunks);
+    int rc = check_launch("feather_flash_attn_fp8");
+    if (!ZS || rc != FEATHER_OK) return rc;
+    return launch_key_range_merge(a, D, n_kchunks, s);
 }
 
 // Workgroup shapes.  A wave of the d = 64 kernel owns 64 queries.  Staging a K/V tile into LDS is
@@ -977,12 +1018,13 @@ static int launch_attn64_wide(const AttnArgs &a, hipStream_t s) {
 // eight waves (twice the queries per staged tile, two waves per SIMD from one workgroup to overlap
 // the barrier-separated phases) are faster wherever the coarser grid still covers the chip's 256 CUs;
 // d = 256 takes eight waves at every length.
-// Key ranges over workgroups (fixed-length, non-causal heads of 128 dims and more): the number of ranges the
+// Key ranges over workgroups (fixed-length, non-causal heads of 64 dims and more): the number of ranges the
 // finest workgroup shape of head dim d is cut into, doubled while the grid still fits the 256 CUs in one pass
 // and a range keeps at least four key tiles.  1 = the plain kernel.
 static int pick_key_chunks(int64_t d, int64_t n_heads, int64_t L) {
     int64_t queries, bn;
     switch (d) {
+        case 64: queries = 256; bn = 64; break;
         case 128: queries = 128; bn = 64; break;
         case 256: queries = 64; bn = 64; break;
         case 512: queries = 64; bn = 32; break;
@@ -1014,6 +1056,8 @@ static int dispatch_attn(const AttnArgs &a, int64_t d, hipStream_t s) {
         case 64:   // all four query blocks of a wave share every K fragment
             // eight waves halve the staging work per query (-2 % time); a causal tile of 512 queries
             // would idle its early waves through too many masked key tiles
+            if constexpr (!VC)
+                if (zs > 1) return launch_attn64_wide<MODE, false, 4, 2, true>(a, s, zs);
             if (!a.causal && fills_chip(512)) return launch_attn64_wide<MODE, VC, 8, 1>(a, s);
             return launch_attn64_wide<MODE, VC, 4, 2>(a, s);
         case 128:

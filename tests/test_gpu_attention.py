@@ -64,6 +64,10 @@ def test_flash_attention_vs_oracle(dev, orc, mode, heads, L, d):
     ("E4M3", 2, 512, 256, "mask", 2), ("E5M2", 1, 1000, 256, "mask", 4), ("E4M3", 1, 1000, 256, "reference", 4),
     ("E4M3", 1, 300, 512, "mask", 2), ("E5M2", 2, 530, 512, "mask", 4), ("E4M3", 1, 530, 512, "reference", 4),
     ("E5M2", 2, 1100, 128, "mask", 4), ("E4M3", 3, 600, 128, "mask", 2), ("E4M3", 8, 1024, 512, "mask", 2),
+    # d = 64: the reference's own call shape, one head (bench_attention.py:13-14: one head of 128 .. 8192 rows) -- 32
+    # workgroups without the key ranges
+    ("E5M2", 1, 8192, 64, "mask", 8), ("E4M3", 2, 3000, 64, "mask", 8), ("E5M2", 1, 1000, 64, "reference", 4),
+    ("E4M3", 1, 2100, 64, "reference", 8),
 ])
 def test_flash_attention_key_ranges_over_workgroups(dev, orc, mode, heads, L, d, tail, ranges):
     """Few short wide heads: with a workspace the key loop of every query tile is cut into `ranges` ranges that

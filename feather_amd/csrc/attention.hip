@@ -1018,22 +1018,31 @@ static int launch_attn64_wide(const AttnArgs &a, hipStream_t s, int n_kchunks = 
 // eight waves (twice the queries per staged tile, two waves per SIMD from one workgroup to overlap
 // the barrier-separated phases) are faster wherever the coarser grid still covers the chip's 256 CUs;
 // d = 256 takes eight waves at every length.
-// Key ranges over workgroups (fixed-length, non-causal heads of 64 dims and more): the number of ranges the
-// finest workgroup shape of head dim d is cut into, doubled while the grid still fits the 256 CUs in one pass
-// and a range keeps at least four key tiles.  1 = the plain kernel.
+// Key ranges over workgroups (fixed-length, non-causal heads of 64 dims and more): the number of ranges (1, 2, 4
+// or 8; 1 = the plain kernel) the finest workgroup shape of head dim d is cut into.  A cost model in nanoseconds:
+// the key loop of a workgroup at its measured time per tile, against the merge kernel (launch and one round trip,
+// then the partial results written, read back and the output written at ~4 TB/s); the grid stays within one pass
+// over the 256 CUs.
 static int pick_key_chunks(int64_t d, int64_t n_heads, int64_t L) {
-    int64_t queries, bn;
+    int64_t queries, bn, tile_ns;
     switch (d) {
-        case 64: queries = 256; bn = 64; break;
-        case 128: queries = 128; bn = 64; break;
-        case 256: queries = 64; bn = 64; break;
-        case 512: queries = 64; bn = 32; break;
+        case 64: queries = 256; bn = 64; tile_ns = 1250; break;
+        case 128: queries = 128; bn = 64; tile_ns = 1900; break;
+        case 256: queries = 64; bn = 64; tile_ns = 2200; break;
+        case 512: queries = 64; bn = 32; tile_ns = 2800; break;
         default: return 1;
     }
     const int64_t wgs = (L + queries - 1) / queries * n_heads, tiles = (L + bn - 1) / bn;
-    int z = 1;
-    while (z < kMaxKeyChunks && wgs * z * 2 <= 256 && tiles / (z * 2) >= 4) z *= 2;
-    return z;
+    int best = 1;
+    int64_t best_ns = tiles * tile_ns;
+    for (int z = 2; z <= kMaxKeyChunks && wgs * z <= 256 && z <= tiles; z *= 2) {
+        const int64_t ns = (tiles + z - 1) / z * tile_ns + 3500 + (2 * z + 1) * n_heads * L * d * 4 / 4000;
+        if (ns + 500 < best_ns) {
+            best = z;
+            best_ns = ns;
+        }
+    }
+    return best;
 }
 
 template <int MODE, bool VC>

@@ -342,6 +342,7 @@ def test_entry_points_replay_in_a_graph():
     M, K = 512, 1024
     mp, vp = feather.pack_fp8_tensor(rn(M, K).half(), mode="E4M3"), feather.pack_fp8_tensor(rn(K).half(), mode="E4M3")
     qkv = [feather.pack_fp8_tensor(rn(2, 256, 64).half(), mode="E5M2").view(2, 256, 16) for _ in range(3)]
+    qkv1 = [feather.pack_fp8_tensor(rn(1, 2048, 64).half(), mode="E5M2").view(2048, 16) for _ in range(3)]   # one head: key ranges + merge
     cfg = DecoderConfig(n_layers=2, hidden=256, n_q_heads=4, n_kv_heads=2, head_dim=64, inter=512, vocab=200)
     B, max_blocks = 3, 48                                      # contexts up to 768: two attention splits
     dec = PackedDecoder(cfg, random_weights(cfg, seed=1), n_blocks=B * max_blocks, max_blocks=max_blocks, mode="E4M3", device=dev)
@@ -357,9 +358,10 @@ def test_entry_points_replay_in_a_graph():
         y = feather.gemv(mp, vp, original_shape=(M, K), mode="E4M3")
         d = feather.dot(mp, mp, mode="E4M3")
         a = feather.flash_attention_fp8_acc_fp32_gpu(qkv[0], qkv[1], qkv[2], 256, 16, mode="E5M2", causal=True)
+        a1 = feather.flash_attention_fp8_e5m2_acc_fp32_gpu(qkv1[0], qkv1[1], qkv1[2], 2048, 16)   # allocates its workspace from torch's pool
         p = paged_attention_fp8_acc_fp32_gpu(q1, dec.layers[0]["k_cache"], dec.layers[0]["v_cache"], bt, ctx, mode="E4M3")
         lg = dec.step(tok, bt, ctx)
-        return y, d, a, p, lg
+        return y, d, a, a1, p, lg
 
     caches0 = [(lay["k_cache"].clone(), lay["v_cache"].clone()) for lay in dec.layers]
     def reset():

@@ -146,12 +146,14 @@ int feather_dot_fp16(const void *x1, const void *x2, void *out_f32, void *scratc
 int feather_flash_attn_fp8(const void *q, const void *k, const void *v, void *out_f32, int64_t n_heads, int64_t L,
                            int64_t d, int64_t kv_group, int mode, float scale, int tail, void *stream);
 
-/* The same attention with an optional device workspace.  Short sequences of few wide heads make a grid that leaves
- * most of the 256 CUs idle (8 heads x 1024 rows at d = 512: 128 workgroups); with a workspace of
- * feather_flash_attn_workspace_bytes(n_heads, L, d) bytes (0: the shape does not profit) the key loop of every query
- * tile is cut into 2 or 4 ranges that run as separate workgroups and a second small kernel combines them (same
- * result to the rounding of the fp32 additions).  workspace == NULL, or a workspace smaller than asked for, runs
- * fewer ranges or the plain kernel; nothing is kept in the workspace between calls.  No reference counterpart
+/* The same attention with an optional device workspace.  One head, or a few short wide heads, make a grid that leaves
+ * most of the 256 CUs idle (the reference function is one head, attention.py:110-179: 8192 rows at d = 64 are 32
+ * workgroups here; 8 heads x 1024 rows at d = 512 are 128).  With a workspace of
+ * feather_flash_attn_workspace_bytes(n_heads, L, d) bytes (0: the shape does not profit; d >= 64) the key loop of every
+ * query tile is cut into 2, 4 or 8 ranges that run as separate workgroups, and a second small kernel combines them
+ * (same result up to the rounding of P against another reference point and of the fp32 additions; identical from call
+ * to call).  workspace == NULL, or a workspace smaller than asked for, runs fewer ranges or the plain kernel; nothing
+ * is kept in the workspace between calls, and calls that share a workspace must not overlap.  No reference counterpart
  * (the reference launches one program per 64 queries of one head, attention.py:172-179). */
 int64_t feather_flash_attn_workspace_bytes(int64_t n_heads, int64_t L, int64_t d);
 int feather_flash_attn_fp8_ws(const void *q, const void *k, const void *v, void *out_f32, void *workspace,

@@ -108,6 +108,25 @@ def test_flash_attention_key_ranges_over_workgroups(dev, orc, mode, heads, L, d,
         assert _nerr(o, plain) <= 8e-4
 
 
+@pytest.mark.parametrize("mode,d,L", [("E4M3", 128, 700), ("E5M2", 64, 1500), ("E4M3", 512, 400)])
+def test_flash_attention_key_ranges_with_grouped_kv_heads(dev, orc, mode, d, L):
+    """Key ranges over workgroups with four query heads on two K/V heads: the partial results are indexed by query
+    head, the K/V rows by the shared head."""
+    from feather_amd import _native as N
+    from feather_amd.routines.attention import flash_attention_fp8_acc_fp32_gpu
+    heads, group = 4, 2
+    assert int(N.lib().feather_flash_attn_workspace_bytes(heads, L, d)) > 0
+    rng = np.random.default_rng(d + L)
+    q, _, _ = _qkv(rng, heads, L, d, mode, orc)
+    _, k, v = _qkv(rng, heads // group, L, d, mode, orc)
+    got = flash_attention_fp8_acc_fp32_gpu(_dev_words(q, dev), _dev_words(k, dev), _dev_words(v, dev), L, d // 4, mode=mode,
+                                           kv_group=group).cpu().numpy().reshape(heads, L, d)
+    per = L * d // 4
+    k_rep = np.concatenate([k.reshape(-1)[(h // group) * per:(h // group + 1) * per] for h in range(heads)])
+    v_rep = np.concatenate([v.reshape(-1)[(h // group) * per:(h // group + 1) * per] for h in range(heads)])
+    assert _nerr(got, orc.attention_f64_np(q, k_rep, v_rep, L, d, mode)) <= TOL
+
+
 @pytest.mark.parametrize("mode", ["E4M3", "E5M2"])
 @pytest.mark.parametrize("heads,L,d", [(8, 1024, 512), (1, 300, 512), (2, 530, 512), (8, 1024, 256), (8, 1024, 128),
                                          (8, 2048, 64), (4, 600, 32)])

@@ -282,11 +282,11 @@ static int launch_gemv_fast(const void *m, const void *v, float *out, int64_t M,
             hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(WAVES * kWave), lds, s, (const uint8_t *)m,
                                (const uint32_t *)vk, out, (int)M, K, (int)k0, kc, (int)rows_per_wg, k0 > 0 ? 1 : 0);
         };
-        // E4M3 with rows under 16 steps loses ~1 % with it (measured at K = 8192), except rows of four steps on
-        // more workgroups than are resident at once (K = 4096: 16384 rows 14.6 -> 13.2 us, 8192 rows 8.6 -> 8.2 us,
-        // 4096 rows 5.3 -> 5.6 us); the fetch uses 128-bit loads
-        const bool early = EARLY && aligned(vk, 16) &&
-                           (MODE == FEATHER_E5M2 || kc >= 16 * kStep || (kc <= 4 * kStep && M >= 8192));
+        // E4M3 rows under 16 steps gain from it only on more workgroups than are resident at once, i.e. from 8192 rows
+        // on (K = 4096: 16384 rows 14.6 -> 13.2 us, 8192 rows 8.6 -> 8.2 us; K = 8192: 8192 rows 13.7 -> 13.3 us, 16384
+        // rows 24.0 -> 23.5 us) and lose below (4096 rows: K = 4096 5.3 -> 5.6 us, K = 8192 7.9 -> 8.2 us); the fetch
+        // uses 128-bit loads
+        const bool early = EARLY && aligned(vk, 16) && (MODE == FEATHER_E5M2 || kc >= 16 * kStep || M >= 8192);
         if (kc % kStep == 0) {
             if (early) go(gemv_fp8_kernel<MODE, RPW, U, WAVES, true, EARLY>);
             else go(gemv_fp8_kernel<MODE, RPW, U, WAVES, true, false>);

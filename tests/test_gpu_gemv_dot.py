@@ -25,6 +25,12 @@ def _nerr(got, want):
     return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
 
 
+
+def _host_decode(words: torch.Tensor, mode: str, orc) -> torch.Tensor:
+    """Packed words copied to the host and decoded there by the oracle's table (kernel semantics); float64 on the CPU."""
+    return torch.from_numpy(orc.decode_np(words.reshape(-1).view(torch.int32).cpu().numpy().view(np.uint32), mode))
+
+
 @pytest.mark.parametrize("mode", ["E5M2", "E4M3"])
 def test_gemv_docstring_known_answer(dev, kats, mode):
     import feather_amd as feather
@@ -170,10 +176,10 @@ def test_gemv_batched_vs_oracle(dev, orc, mode, M, K, nvec):
 
 
 @pytest.mark.parametrize("M,K", [(32000, 2048), (11264, 2048), (2048, 5632), (2560, 2048)])
-def test_gemv_batched_decode_shapes_vs_fp64_math(dev, M, K):
-    """The weight shapes of the TinyLlama-shaped decode step at batch 32, E4M3: against a float64
-    matmul of the operands decoded by the HIP unpack kernel on the device (the scalar oracle is too slow
-    here; the unpack kernel is held bit-exact to the oracle's decode on all 256 codes by test_gpu_pack.py)."""
+def test_gemv_batched_decode_shapes_vs_fp64_math(dev, orc, M, K):
+    """The weight shapes of the TinyLlama-shaped decode step at batch 32, E4M3: against a float64 matmul of the
+    operands, whose packed words are copied to the host and decoded there by the oracle's table (the scalar
+    oracle's own loop is too slow at these sizes)."""
     import feather_amd as feather
     from feather_amd.routines.gemv import gemv_fp8_batched_acc_fp32_gpu
     g = torch.Generator(device=dev).manual_seed(M + K)
@@ -181,15 +187,15 @@ def test_gemv_batched_decode_shapes_vs_fp64_math(dev, M, K):
     x16 = torch.randn(32, K, generator=g, device=dev).half()
     wp, xp = feather.pack_fp8_tensor(w16, mode="E4M3"), feather.pack_fp8_tensor(x16, mode="E4M3")
     out = gemv_fp8_batched_acc_fp32_gpu(wp, xp, (M, K), 32, "E4M3")
-    wd = feather.unpack_fp8_tensor(wp, mode="E4M3", semantics="kernel").view(M, K).double()
-    xd = feather.unpack_fp8_tensor(xp, mode="E4M3", semantics="kernel").view(32, K).double()
+    wd = orc.decode_np(wp.view(torch.int32).cpu().numpy().view(np.uint32).reshape(-1), "E4M3").reshape(M, K)
+    xd = orc.decode_np(xp.view(torch.int32).cpu().numpy().view(np.uint32).reshape(-1), "E4M3").reshape(32, K)
     want = xd @ wd.T
     assert out.shape == (32, M)
-    assert ((out.double() - want).abs().max() / want.abs().max()).item() <= TOL
+    assert np.abs(out.cpu().numpy().astype(np.float64) - want).max() / np.abs(want).max() <= TOL
 
 
 @pytest.mark.parametrize("seed", range(10))
-def test_gemv_batched_random_shapes(dev, seed):
+def test_gemv_batched_random_shapes(dev, orc, seed):
     """Seeded random (mode, M, K, nvec) draws against a float64 matmul of the decoded operands on
     the device: the launcher switches between one and two K groups per workgroup and the
     per-vector path on K, M and the vector count; codes are raw random bytes (every code occurs,
@@ -208,16 +214,15 @@ def test_gemv_batched_random_shapes(dev, seed):
         return torch.from_numpy(b.view(np.int32).copy()).to(dev).view(torch.uint32)
     wp, xp = codes(M * K), codes(nvec * K)
     out = gemv_fp8_batched_acc_fp32_gpu(wp, xp, (M, K), nvec, mode)
-    wd = feather.unpack_fp8_tensor(wp, mode=mode, semantics="kernel").view(M, K).double()
-    xd = feather.unpack_fp8_tensor(xp, mode=mode, semantics="kernel").view(nvec, K).double()
+    wd, xd = _host_decode(wp, mode, orc).view(M, K), _host_decode(xp, mode, orc).view(nvec, K)
     want = xd @ wd.T
     scale = (xd.abs() @ wd.abs().T).max()               # cancellation-free error scale of the fp32 sums
     assert out.shape == (nvec, M)
-    assert ((out.double() - want).abs().max() / scale).item() <= 1e-5
+    assert ((out.double().cpu() - want).abs().max() / scale).item() <= 1e-5
 
 
 @pytest.mark.parametrize("seed", range(14))
-def test_gemv_random_shapes(dev, seed):
+def test_gemv_random_shapes(dev, orc, seed):
     """Seeded random (mode, M, K) draws for the single-vector GEMV against a float64 matvec of the
     decoded operands on the device: rows shorter and longer than four 1 KiB steps, ragged last steps,
     rows longer than one 32768-code vector chunk, row counts that are not a multiple of a workgroup's
@@ -235,12 +240,11 @@ def test_gemv_random_shapes(dev, seed):
     wp, xp = codes(M * K), codes(K)
     print(f"seed {seed}: {mode} M {M} K {K}", flush=True)
     out = feather.gemv(wp, xp, original_shape=(M, K), mode=mode)
-    wd = feather.unpack_fp8_tensor(wp, mode=mode, semantics="kernel").view(M, K).double()
-    xd = feather.unpack_fp8_tensor(xp, mode=mode, semantics="kernel").view(K).double()
+    wd, xd = _host_decode(wp, mode, orc).view(M, K), _host_decode(xp, mode, orc).view(K)
     want = wd @ xd
     scale = (wd.abs() @ xd.abs()).max()                 # cancellation-free error scale of the fp32 sums
     assert out.shape == (M,)
-    assert ((out.double() - want).abs().max() / scale).item() <= 1e-5
+    assert ((out.double().cpu() - want).abs().max() / scale).item() <= 1e-5
 
 
 @pytest.mark.parametrize("mode", ["E5M2", "E4M3"])
@@ -347,11 +351,10 @@ def test_gemv_config_size_8192_vs_oracle(dev, orc):
     assert np.array_equal(mw[rows], orc.pack_fp8(m.numpy()[rows], "E5M2").reshape(len(rows), K // 4))   # packing bit-exact
     vw = vp.view(torch.int32).cpu().numpy().view(np.uint32)
     want = orc.gemv(np.ascontiguousarray(mw[rows]).reshape(-1), vw, len(rows), K, "E5M2", acc64=True)
-    full = torch.mv(feather.unpack_fp8_tensor(mp, mode="E5M2", semantics="kernel").view(M, K).double(),
-                    feather.unpack_fp8_tensor(vp, mode="E5M2", semantics="kernel").double())
+    full = torch.mv(_host_decode(mp, "E5M2", orc).view(M, K), _host_decode(vp, "E5M2", orc)[:K])   # every row, float64 on the host
     scale = full.abs().max().item()
     assert np.abs(out.cpu().numpy()[rows] - want).max() / scale <= 1e-5
-    assert ((out.double() - full).abs().max() / scale).item() <= 1e-5
+    assert ((out.double().cpu() - full).abs().max() / scale).item() <= 1e-5
 
 
 @pytest.mark.parametrize("n", [2, 1001, 1 << 20])

@@ -117,10 +117,10 @@ def test_gemv_swiglu_epilogue_bit_exact_codes(dev, orc, mode, inter, K, nvec):
     act, f = gemv_fp8_batched_swiglu(wp, xp, inter, K, nvec, mode=mode, return_f32=True)
     f = f.cpu().numpy()
     assert np.array_equal(_np_words(act).reshape(-1), decode_ref.quant_codes(f, mode))
-    wd = feather.unpack_fp8_tensor(wp, mode=mode, semantics="kernel").view(2 * inter, K).double()
-    xd = feather.unpack_fp8_tensor(xp, mode=mode, semantics="kernel").view(nvec, K).double()
+    wd = torch.from_numpy(orc.decode_np(_np_words(wp).reshape(-1), mode)).view(2 * inter, K)      # decoded on the host
+    xd = torch.from_numpy(orc.decode_np(_np_words(xp).reshape(-1), mode)).view(nvec, K)
     gu = xd @ wd.T
-    want = (torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]).cpu().numpy()
+    want = (torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]).numpy()
     assert np.abs(f - want).max() <= 1e-3 * np.abs(want).max()
     if (inter, K) == (96, 256):                                 # a shape the scalar oracle covers: its own GEMV, too
         gu_o = orc.gemv(_np_words(wp), _np_words(xp)[: K // 4], 2 * inter, K, mode, acc64=True)
